@@ -1,0 +1,170 @@
+/*
+ * motifcl_amd.h -- C ABI of the MI355X (gfx950) compact-counter update library.
+ *
+ * Every entry point takes plain device pointers with their byte sizes, scalar
+ * arguments and a HIP stream (hipStream_t passed as void*, NULL = the default
+ * stream).  Work is enqueued on that stream and the call returns without
+ * waiting.  Return value: 0 (MCC_OK) on success, a negative MCC_E_* code on
+ * failure; mcc_last_error() then returns the message for the calling thread.
+ * Validation failures never enqueue work and never throw -- the convention of
+ * the reference's VulkanOpResult{success,error}
+ * (include/motifcl/runtime/vulkan_backend.hpp:80-84).
+ *
+ * Data layout (kernels/compact_counter.cl:1-5):
+ *   state  u8  [out, in/4, 3]  four 6-bit codes per 3 bytes, little-endian
+ *                              24-bit word c0 | c1<<6 | c2<<12 | c3<<18
+ *   scale  f32 [out]           per-row weight scale
+ *   v      f32 [out]           per-row RMS second moment
+ *   grad_w f32 [out, in]       dense weight gradient, row-major
+ *   x      f32 [batch, in]     layer input, row-major
+ *   grad_out f32 [batch, out]  upstream gradient, row-major
+ */
+#ifndef MOTIFCL_AMD_H
+#define MOTIFCL_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MCC_OK 0
+#define MCC_E_INVALID (-1) /* argument validation failed; nothing was enqueued */
+#define MCC_E_RUNTIME (-2) /* a HIP call failed */
+
+/* Message of the last failure on this thread ("" if none). */
+const char* mcc_last_error(void);
+
+/* Name and architecture of the current HIP device, e.g. "AMD Instinct MI355X (gfx950)".
+ * Replaces VulkanOpResult::device_name. */
+const char* mcc_device_name(void);
+
+/*
+ * Update-only step: the optimizer step for a supplied dense weight gradient.
+ * Replaces CounterStateLinear::apply_update_seed
+ * (src/nn/compact_counter.cpp:113-156: counter_row_stats_f32 ->
+ * counter_apply_update_f32 -> copy_f32; kernels/compact_counter.cl:59-139).
+ * Mutates state, scale and v in place.  Results are bit-identical to the
+ * reference arithmetic evaluated in IEEE-754 binary32 without contraction.
+ */
+int mcc_compact_counter_apply_update_dense(
+    void* stream,
+    uint8_t* state, size_t state_nbytes,
+    float* scale, size_t scale_nbytes,
+    float* v, size_t v_nbytes,
+    const float* grad_w, size_t grad_w_nbytes,
+    size_t C, size_t in_features, size_t out_features,
+    float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
+
+/*
+ * Bytes of transient workspace mcc_compact_counter_apply_update_fused needs
+ * for the given shape (0 on invalid dimensions).
+ */
+size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out_features,
+                                                  size_t batch);
+
+/*
+ * Fused step: weight-gradient contraction grad_w = grad_out^T . x on the fp32
+ * matrix cores followed by the counter update.
+ * Replaces run_vulkan_compact_counter_apply_update_fused
+ * (include/motifcl/runtime/vulkan_backend.hpp:733-749,
+ *  src/runtime/vulkan_backend.cpp:8475-8578) and the OpenCL twin in
+ * CounterStateLinear::apply_update_backward (src/nn/compact_counter.cpp:158-231).
+ * The reference's scale_new/denom scratch buffers are not needed; instead the
+ * caller lends `workspace` (>= mcc_compact_counter_fused_workspace_nbytes).
+ * grad_w differs from the reference's sequential fp32 sum only by summation
+ * order (relative error <= 1e-4 of the row norm); given that grad_w the counter
+ * arithmetic is the same as in the dense entry point.
+ */
+int mcc_compact_counter_apply_update_fused(
+    void* stream,
+    uint8_t* state, size_t state_nbytes,
+    float* scale, size_t scale_nbytes,
+    float* v, size_t v_nbytes,
+    const float* grad_out, size_t grad_out_nbytes,
+    const float* x, size_t x_nbytes,
+    void* workspace, size_t workspace_nbytes,
+    size_t C, size_t in_features, size_t out_features, size_t batch,
+    float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
+
+/*
+ * c[m,n] = a[k,m]^T . b[k,n], fp32, row-major.
+ * Replaces matmul_transpose_a (include/motifcl/ops/matmul.hpp:8,
+ * src/ops/matmul.cpp:1416-1418), the producer of the dense weight gradient
+ * (grad_w = matmul_transpose_a(grad_out, x), tests/test_memory_truth_gate.cpp:49).
+ */
+int mcc_matmul_transpose_a_f32(
+    void* stream,
+    const float* a, size_t a_nbytes,
+    const float* b, size_t b_nbytes,
+    float* c, size_t c_nbytes,
+    size_t k, size_t m, size_t n);
+
+/*
+ * weight[out,in] = scale[row] * t(state).
+ * Replaces run_vulkan_compact_counter_decode_weight
+ * (include/motifcl/runtime/vulkan_backend.hpp:713-719,
+ *  src/runtime/vulkan_backend.cpp:8603-8660; kernels/compact_counter.cl:39-55).
+ */
+int mcc_compact_counter_decode_weight(
+    void* stream,
+    const uint8_t* state, size_t state_nbytes,
+    const float* scale, size_t scale_nbytes,
+    float* weight, size_t weight_nbytes,
+    size_t in_features, size_t out_features, size_t C);
+
+/*
+ * out[batch,out] = x[batch,in] . W(state)^T with the ternary weights decoded
+ * from the packed state inside the contraction (no dense weight buffer).
+ * Replaces run_vulkan_compact_counter_forward_u8
+ * (include/motifcl/runtime/vulkan_backend.hpp:722-730,
+ *  src/runtime/vulkan_backend.cpp:8662-8725).
+ */
+int mcc_compact_counter_forward_u8(
+    void* stream,
+    const float* x, size_t x_nbytes,
+    const uint8_t* state, size_t state_nbytes,
+    const float* scale, size_t scale_nbytes,
+    float* out, size_t out_nbytes,
+    size_t batch, size_t in_features, size_t out_features, size_t C);
+
+/*
+ * grad_x[batch,in] = grad_out[batch,out] . W(state), decoded in-kernel.
+ * Replaces run_vulkan_compact_counter_backward_input_u8
+ * (include/motifcl/runtime/vulkan_backend.hpp:750-758,
+ *  src/runtime/vulkan_backend.cpp:8727-8803; kernels/compact_counter.cl:248-269).
+ */
+int mcc_compact_counter_backward_input_u8(
+    void* stream,
+    const uint8_t* state, size_t state_nbytes,
+    const float* scale, size_t scale_nbytes,
+    const float* grad_out, size_t grad_out_nbytes,
+    float* grad_x, size_t grad_x_nbytes,
+    size_t batch, size_t in_features, size_t out_features, size_t C);
+
+/*
+ * Device-resident storage.  Replaces the pooled VulkanRuntime::create_buffer /
+ * Storage allocator (src/runtime/vulkan_backend.cpp:4663-4719,6462-6510;
+ * src/tensor/storage.cpp:35-79): freed blocks are kept in power-of-two buckets
+ * and reused; mcc_device_pool_clear returns them to the driver.  The byte
+ * counters mirror device_bytes_current/peak (src/runtime/buffer.cpp:16-30).
+ */
+int mcc_device_alloc(void** ptr, size_t nbytes);
+int mcc_device_free(void* ptr);
+int mcc_device_pool_clear(void);
+size_t mcc_device_bytes_current(void);
+size_t mcc_device_bytes_peak(void);
+void mcc_device_bytes_reset_peak(void);
+int mcc_memcpy_h2d(void* stream, void* dst, const void* src, size_t nbytes);
+int mcc_memcpy_d2h(void* stream, void* dst, const void* src, size_t nbytes);
+int mcc_memset_zero(void* stream, void* dst, size_t nbytes);
+/* Waits for everything enqueued on `stream` (Backend::finish,
+ * src/runtime/backend.cpp:328-331). */
+int mcc_stream_synchronize(void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MOTIFCL_AMD_H */

@@ -1,0 +1,394 @@
+// C ABI of the library: argument validation, error reporting and device
+// storage.  Validation mirrors the reference's Vulkan host wrappers
+// (src/runtime/vulkan_backend.cpp:8497-8521, 8603-8650, 8662-8712, 8727-8786):
+// failures are reported, never thrown, and enqueue nothing.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <limits>
+#include <map>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/motifcl_amd.h"
+#include "launch.hpp"
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const std::string& message) {
+    g_error = message;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    return fail(MCC_E_RUNTIME, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+constexpr size_t kIntMax = static_cast<size_t>(std::numeric_limits<int>::max());
+
+// Shared shape/codec checks.  `what` names the operation in messages.
+bool check_codec(const char* what, size_t C, size_t in_features, size_t out_features) {
+    if (in_features == 0 || out_features == 0) {
+        g_error = std::string(what) + " requires non-zero dimensions";
+        return false;
+    }
+    if (in_features % 4 != 0) {
+        g_error = std::string(what) + " requires in_features divisible by 4";
+        return false;
+    }
+    if (C == 0 || 3 * (2 * C - 1) > 64) {
+        g_error = std::string(what) + " C is out of 6-bit range";
+        return false;
+    }
+    if (in_features > kIntMax || out_features > kIntMax ||
+        out_features > kIntMax / in_features) {
+        g_error = std::string(what) + " dimensions exceed the 32-bit element index of the state encoding";
+        return false;
+    }
+    return true;
+}
+
+// ---- pooled device storage -------------------------------------------------
+struct Pool {
+    std::mutex mu;
+    std::map<size_t, std::vector<void*>> free_blocks;   // bucket bytes -> cached blocks
+    std::unordered_map<void*, size_t> live;             // block -> bucket bytes
+    size_t cached_bytes = 0;
+};
+Pool& pool() {
+    static Pool p;
+    return p;
+}
+std::atomic<size_t> g_bytes_current{0};
+std::atomic<size_t> g_bytes_peak{0};
+constexpr size_t kPoolMaxCachedBytes = size_t(2) << 30;  // cap as in vulkan_backend.cpp:6462-6510
+
+size_t bucket_of(size_t nbytes) {
+    size_t b = 256;
+    while (b < nbytes) b <<= 1;
+    return b;
+}
+
+__global__ void fill_zero_kernel(uint8_t* dst, size_t nbytes) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nbytes; i += stride) dst[i] = 0;
+}
+
+void track_alloc(size_t n) {
+    const size_t cur = g_bytes_current.fetch_add(n) + n;
+    size_t prev = g_bytes_peak.load();
+    while (cur > prev && !g_bytes_peak.compare_exchange_weak(prev, cur)) {
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mcc_last_error(void) { return g_error.c_str(); }
+
+const char* mcc_device_name(void) {
+    static thread_local std::string name;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+        name = "";
+        return name.c_str();
+    }
+    name = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+    return name.c_str();
+}
+
+int mcc_compact_counter_apply_update_dense(void* stream, uint8_t* state, size_t state_nbytes,
+                                           float* scale, size_t scale_nbytes, float* v,
+                                           size_t v_nbytes, const float* grad_w,
+                                           size_t grad_w_nbytes, size_t C, size_t in_features,
+                                           size_t out_features, float lr, float lr_scale,
+                                           float rms_beta, float rms_eps, uint32_t seed) {
+    const char* what = "compact-counter update";
+    if (!check_codec(what, C, in_features, out_features)) return MCC_E_INVALID;
+    if (!std::isfinite(lr)) return fail(MCC_E_INVALID, "compact-counter update requires finite lr");
+    if (!std::isfinite(lr_scale)) return fail(MCC_E_INVALID, "compact-counter update requires finite lr_scale");
+    if (!std::isfinite(rms_beta)) return fail(MCC_E_INVALID, "compact-counter update requires finite rms_beta");
+    if (!std::isfinite(rms_eps) || rms_eps < 0.0f)
+        return fail(MCC_E_INVALID, "compact-counter update requires non-negative finite rms_eps");
+    if (!state || !scale || !v || !grad_w) return fail(MCC_E_INVALID, "compact-counter update received a null buffer");
+    const size_t n_groups = out_features * (in_features / 4);
+    if (state_nbytes < n_groups * 3) return fail(MCC_E_INVALID, "compact-counter update state buffer is too small");
+    if (scale_nbytes < out_features * sizeof(float) || v_nbytes < out_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter update per-row buffer is too small");
+    if (grad_w_nbytes < out_features * in_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter update gradient buffer is too small");
+    if (reinterpret_cast<uintptr_t>(grad_w) % alignof(float) || reinterpret_cast<uintptr_t>(scale) % alignof(float) ||
+        reinterpret_cast<uintptr_t>(v) % alignof(float))
+        return fail(MCC_E_INVALID, "compact-counter update float buffers must be 4-byte aligned");
+    const hipError_t e = mcc::launch_update_dense(static_cast<hipStream_t>(stream), state, scale, v, grad_w,
+                                                  (int)C, (int)in_features, (int)out_features, lr,
+                                                  lr_scale, rms_beta, rms_eps, seed);
+    if (e != hipSuccess) return hip_fail(e, "compact-counter update launch failed");
+    return MCC_OK;
+}
+
+size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out_features,
+                                                  size_t batch) {
+    if (in_features == 0 || out_features == 0 || batch == 0) return 0;
+    if (out_features > std::numeric_limits<size_t>::max() / sizeof(float) / in_features) return 0;
+    return out_features * in_features * sizeof(float);
+}
+
+int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t state_nbytes,
+                                           float* scale, size_t scale_nbytes, float* v,
+                                           size_t v_nbytes, const float* grad_out,
+                                           size_t grad_out_nbytes, const float* x, size_t x_nbytes,
+                                           void* workspace, size_t workspace_nbytes, size_t C,
+                                           size_t in_features, size_t out_features, size_t batch,
+                                           float lr, float lr_scale, float rms_beta, float rms_eps,
+                                           uint32_t seed) {
+    const char* what = "compact-counter fused update";
+    if (batch == 0) return fail(MCC_E_INVALID, "compact-counter fused update requires non-zero dimensions");
+    if (!check_codec(what, C, in_features, out_features)) return MCC_E_INVALID;
+    if (batch > kIntMax) return fail(MCC_E_INVALID, "compact-counter fused update batch exceeds 2^31-1");
+    if (!std::isfinite(lr)) return fail(MCC_E_INVALID, "compact-counter fused update requires finite lr");
+    if (!std::isfinite(lr_scale)) return fail(MCC_E_INVALID, "compact-counter fused update requires finite lr_scale");
+    if (!std::isfinite(rms_beta)) return fail(MCC_E_INVALID, "compact-counter fused update requires finite rms_beta");
+    if (!std::isfinite(rms_eps) || rms_eps < 0.0f)
+        return fail(MCC_E_INVALID, "compact-counter fused update requires non-negative finite rms_eps");
+    if (!state || !scale || !v || !grad_out || !x || !workspace)
+        return fail(MCC_E_INVALID, "compact-counter fused update received a null buffer");
+    const size_t n_groups = out_features * (in_features / 4);
+    if (state_nbytes < n_groups * 3) return fail(MCC_E_INVALID, "compact-counter fused update state buffer is too small");
+    if (scale_nbytes < out_features * sizeof(float) || v_nbytes < out_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter fused update per-row buffer is too small");
+    if (batch > std::numeric_limits<size_t>::max() / sizeof(float) / in_features ||
+        batch > std::numeric_limits<size_t>::max() / sizeof(float) / out_features)
+        return fail(MCC_E_INVALID, "compact-counter fused update activation size overflows size_t");
+    if (grad_out_nbytes < batch * out_features * sizeof(float) || x_nbytes < batch * in_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter fused update activation buffer is too small");
+    if (workspace_nbytes < mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch))
+        return fail(MCC_E_INVALID, "compact-counter fused update workspace is too small");
+    if (reinterpret_cast<uintptr_t>(workspace) % 16)
+        return fail(MCC_E_INVALID, "compact-counter fused update workspace must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(grad_out) % alignof(float) || reinterpret_cast<uintptr_t>(x) % alignof(float) ||
+        reinterpret_cast<uintptr_t>(scale) % alignof(float) || reinterpret_cast<uintptr_t>(v) % alignof(float))
+        return fail(MCC_E_INVALID, "compact-counter fused update float buffers must be 4-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    float* grad_w = static_cast<float*>(workspace);
+    hipError_t e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features);
+    if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
+    e = mcc::launch_update_dense(s, state, scale, v, grad_w, (int)C, (int)in_features, (int)out_features, lr,
+                                 lr_scale, rms_beta, rms_eps, seed);
+    if (e != hipSuccess) return hip_fail(e, "compact-counter fused update launch failed");
+    return MCC_OK;
+}
+
+int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, const float* b,
+                               size_t b_nbytes, float* c, size_t c_nbytes, size_t k, size_t m,
+                               size_t n) {
+    if (k == 0 || m == 0 || n == 0) return fail(MCC_E_INVALID, "matmul_transpose_a requires non-zero dimensions");
+    if (k > kIntMax || m > kIntMax || n > kIntMax)
+        return fail(MCC_E_INVALID, "matmul_transpose_a dimensions exceed 2^31-1");
+    if (!a || !b || !c) return fail(MCC_E_INVALID, "matmul_transpose_a received a null buffer");
+    if (k > std::numeric_limits<size_t>::max() / sizeof(float) / m ||
+        k > std::numeric_limits<size_t>::max() / sizeof(float) / n ||
+        m > std::numeric_limits<size_t>::max() / sizeof(float) / n)
+        return fail(MCC_E_INVALID, "matmul_transpose_a buffer size overflows size_t");
+    if (a_nbytes < k * m * sizeof(float) || b_nbytes < k * n * sizeof(float) || c_nbytes < m * n * sizeof(float))
+        return fail(MCC_E_INVALID, "matmul_transpose_a buffer is too small");
+    if (reinterpret_cast<uintptr_t>(a) % alignof(float) || reinterpret_cast<uintptr_t>(b) % alignof(float) ||
+        reinterpret_cast<uintptr_t>(c) % alignof(float))
+        return fail(MCC_E_INVALID, "matmul_transpose_a buffers must be 4-byte aligned");
+    const hipError_t e = mcc::launch_gemm_tn_f32(static_cast<hipStream_t>(stream), a, b, c, (int)k, (int)m, (int)n);
+    if (e != hipSuccess) return hip_fail(e, "matmul_transpose_a launch failed");
+    return MCC_OK;
+}
+
+int mcc_compact_counter_decode_weight(void* stream, const uint8_t* state, size_t state_nbytes,
+                                      const float* scale, size_t scale_nbytes, float* weight,
+                                      size_t weight_nbytes, size_t in_features, size_t out_features,
+                                      size_t C) {
+    if (!check_codec("compact-counter decode", C, in_features, out_features)) return MCC_E_INVALID;
+    if (!state || !scale || !weight) return fail(MCC_E_INVALID, "compact-counter decode received a null buffer");
+    const size_t groups = out_features * (in_features / 4);
+    if (state_nbytes < groups * 3) return fail(MCC_E_INVALID, "compact-counter state buffer is too small");
+    if (scale_nbytes < out_features * sizeof(float)) return fail(MCC_E_INVALID, "compact-counter scale buffer is too small");
+    if (weight_nbytes < out_features * in_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter weight buffer is too small");
+    const hipError_t e = mcc::launch_decode_weight(static_cast<hipStream_t>(stream), state, scale, weight, (int)C,
+                                                   (int)in_features, (int)out_features);
+    if (e != hipSuccess) return hip_fail(e, "compact-counter decode launch failed");
+    return MCC_OK;
+}
+
+int mcc_compact_counter_forward_u8(void* stream, const float* x, size_t x_nbytes,
+                                   const uint8_t* state, size_t state_nbytes, const float* scale,
+                                   size_t scale_nbytes, float* out, size_t out_nbytes, size_t batch,
+                                   size_t in_features, size_t out_features, size_t C) {
+    if (batch == 0) return fail(MCC_E_INVALID, "compact-counter forward requires non-zero dimensions");
+    if (!check_codec("compact-counter forward", C, in_features, out_features)) return MCC_E_INVALID;
+    if (batch > kIntMax / 16) return fail(MCC_E_INVALID, "compact-counter forward batch is too large");
+    if (!x || !state || !scale || !out) return fail(MCC_E_INVALID, "compact-counter forward received a null buffer");
+    const size_t groups = out_features * (in_features / 4);
+    if (state_nbytes < groups * 3) return fail(MCC_E_INVALID, "compact-counter forward state buffer is too small");
+    if (scale_nbytes < out_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter forward scale buffer is too small");
+    if (batch > std::numeric_limits<size_t>::max() / sizeof(float) / in_features ||
+        batch > std::numeric_limits<size_t>::max() / sizeof(float) / out_features)
+        return fail(MCC_E_INVALID, "compact-counter forward buffer size overflows size_t");
+    if (x_nbytes < batch * in_features * sizeof(float) || out_nbytes < batch * out_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter forward activation buffer is too small");
+    const hipError_t e = mcc::launch_forward(static_cast<hipStream_t>(stream), x, state, scale, out, (int)C,
+                                             (int)batch, (int)in_features, (int)out_features);
+    if (e != hipSuccess) return hip_fail(e, "compact-counter forward launch failed");
+    return MCC_OK;
+}
+
+int mcc_compact_counter_backward_input_u8(void* stream, const uint8_t* state, size_t state_nbytes,
+                                          const float* scale, size_t scale_nbytes,
+                                          const float* grad_out, size_t grad_out_nbytes,
+                                          float* grad_x, size_t grad_x_nbytes, size_t batch,
+                                          size_t in_features, size_t out_features, size_t C) {
+    if (batch == 0) return fail(MCC_E_INVALID, "compact-counter backward-input requires non-zero dimensions");
+    if (!check_codec("compact-counter backward-input", C, in_features, out_features)) return MCC_E_INVALID;
+    if (batch > kIntMax) return fail(MCC_E_INVALID, "compact-counter backward-input batch is too large");
+    if (!state || !scale || !grad_out || !grad_x)
+        return fail(MCC_E_INVALID, "compact-counter backward-input received a null buffer");
+    const size_t groups = out_features * (in_features / 4);
+    if (state_nbytes < groups * 3) return fail(MCC_E_INVALID, "compact-counter state buffer is too small");
+    if (scale_nbytes < out_features * sizeof(float)) return fail(MCC_E_INVALID, "compact-counter scale buffer is too small");
+    if (batch > std::numeric_limits<size_t>::max() / sizeof(float) / in_features ||
+        batch > std::numeric_limits<size_t>::max() / sizeof(float) / out_features)
+        return fail(MCC_E_INVALID, "compact-counter backward-input buffer size overflows size_t");
+    if (grad_out_nbytes < batch * out_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter grad_out buffer is too small");
+    if (grad_x_nbytes < batch * in_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter grad_x buffer is too small");
+    const hipError_t e = mcc::launch_backward_input(static_cast<hipStream_t>(stream), grad_out, state, scale,
+                                                    grad_x, (int)C, (int)batch, (int)in_features,
+                                                    (int)out_features);
+    if (e != hipSuccess) return hip_fail(e, "compact-counter backward-input launch failed");
+    return MCC_OK;
+}
+
+// ---- storage ---------------------------------------------------------------
+int mcc_device_alloc(void** ptr, size_t nbytes) {
+    if (!ptr) return fail(MCC_E_INVALID, "device alloc received a null result pointer");
+    if (nbytes == 0) return fail(MCC_E_INVALID, "cannot allocate zero-byte buffer");
+    const size_t bucket = bucket_of(nbytes);
+    Pool& p = pool();
+    {
+        std::lock_guard<std::mutex> lock(p.mu);
+        auto it = p.free_blocks.find(bucket);
+        if (it != p.free_blocks.end() && !it->second.empty()) {
+            *ptr = it->second.back();
+            it->second.pop_back();
+            p.cached_bytes -= bucket;
+            p.live[*ptr] = bucket;
+            return MCC_OK;
+        }
+    }
+    void* d = nullptr;
+    const hipError_t e = hipMalloc(&d, bucket);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc failed");
+    track_alloc(bucket);
+    {
+        std::lock_guard<std::mutex> lock(p.mu);
+        p.live[d] = bucket;
+    }
+    *ptr = d;
+    return MCC_OK;
+}
+
+int mcc_device_free(void* ptr) {
+    if (!ptr) return MCC_OK;
+    Pool& p = pool();
+    size_t bucket = 0;
+    bool cache = false;
+    {
+        std::lock_guard<std::mutex> lock(p.mu);
+        auto it = p.live.find(ptr);
+        if (it == p.live.end()) return fail(MCC_E_INVALID, "device free of a pointer this library did not allocate");
+        bucket = it->second;
+        p.live.erase(it);
+        if (p.cached_bytes + bucket <= kPoolMaxCachedBytes) {
+            p.free_blocks[bucket].push_back(ptr);
+            p.cached_bytes += bucket;
+            cache = true;
+        }
+    }
+    if (!cache) {
+        const hipError_t e = hipFree(ptr);
+        g_bytes_current.fetch_sub(bucket);
+        if (e != hipSuccess) return hip_fail(e, "hipFree failed");
+    }
+    return MCC_OK;
+}
+
+int mcc_device_pool_clear(void) {
+    Pool& p = pool();
+    std::vector<std::pair<void*, size_t>> blocks;
+    {
+        std::lock_guard<std::mutex> lock(p.mu);
+        for (auto& kv : p.free_blocks)
+            for (void* b : kv.second) blocks.emplace_back(b, kv.first);
+        p.free_blocks.clear();
+        p.cached_bytes = 0;
+    }
+    int rc = MCC_OK;
+    for (auto& b : blocks) {
+        const hipError_t e = hipFree(b.first);
+        g_bytes_current.fetch_sub(b.second);
+        if (e != hipSuccess) rc = hip_fail(e, "hipFree failed");
+    }
+    return rc;
+}
+
+size_t mcc_device_bytes_current(void) { return g_bytes_current.load(); }
+size_t mcc_device_bytes_peak(void) { return g_bytes_peak.load(); }
+void mcc_device_bytes_reset_peak(void) { g_bytes_peak.store(g_bytes_current.load()); }
+
+int mcc_memcpy_h2d(void* stream, void* dst, const void* src, size_t nbytes) {
+    if (nbytes == 0) return MCC_OK;
+    if (!dst || !src) return fail(MCC_E_INVALID, "memcpy received a null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);  // src may be pageable and reused by the caller
+    if (e != hipSuccess) return hip_fail(e, "host-to-device copy failed");
+    return MCC_OK;
+}
+
+int mcc_memcpy_d2h(void* stream, void* dst, const void* src, size_t nbytes) {
+    if (nbytes == 0) return MCC_OK;
+    if (!dst || !src) return fail(MCC_E_INVALID, "memcpy received a null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(e, "device-to-host copy failed");
+    return MCC_OK;
+}
+
+int mcc_memset_zero(void* stream, void* dst, size_t nbytes) {
+    if (nbytes == 0) return MCC_OK;
+    if (!dst) return fail(MCC_E_INVALID, "memset received a null pointer");
+    // a fill kernel rather than hipMemsetAsync, so that the call stays valid under graph capture
+    const unsigned blocks = (unsigned)((nbytes + 255) / 256 < 4096 ? (nbytes + 255) / 256 : 4096);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint8_t*>(dst), nbytes);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "device memset failed");
+    return MCC_OK;
+}
+
+int mcc_stream_synchronize(void* stream) {
+    const hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "stream synchronize failed");
+    return MCC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,76 @@
+"""Loads libmotifcl_amd.so and declares the C ABI of include/motifcl_amd.h for ctypes."""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmotifcl_amd.so")
+
+_vp, _sz, _f, _u32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_uint32
+
+# name -> (restype, argtypes); one entry per declaration in include/motifcl_amd.h
+SIGNATURES = {
+    "mcc_last_error": (ctypes.c_char_p, []),
+    "mcc_device_name": (ctypes.c_char_p, []),
+    "mcc_compact_counter_apply_update_dense": (
+        ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
+    "mcc_compact_counter_fused_workspace_nbytes": (_sz, [_sz, _sz, _sz]),
+    "mcc_compact_counter_apply_update_fused": (
+        ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
+                       _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
+    "mcc_matmul_transpose_a_f32": (ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz]),
+    "mcc_compact_counter_decode_weight": (ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz]),
+    "mcc_compact_counter_forward_u8": (
+        ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _sz]),
+    "mcc_compact_counter_backward_input_u8": (
+        ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _sz]),
+    "mcc_device_alloc": (ctypes.c_int, [ctypes.POINTER(_vp), _sz]),
+    "mcc_device_free": (ctypes.c_int, [_vp]),
+    "mcc_device_pool_clear": (ctypes.c_int, []),
+    "mcc_device_bytes_current": (_sz, []),
+    "mcc_device_bytes_peak": (_sz, []),
+    "mcc_device_bytes_reset_peak": (None, []),
+    "mcc_memcpy_h2d": (ctypes.c_int, [_vp, _vp, _vp, _sz]),
+    "mcc_memcpy_d2h": (ctypes.c_int, [_vp, _vp, _vp, _sz]),
+    "mcc_memset_zero": (ctypes.c_int, [_vp, _vp, _sz]),
+    "mcc_stream_synchronize": (ctypes.c_int, [_vp]),
+}
+
+_lib = None
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def load():
+    """Returns the loaded library; raises LibraryMissing if it has not been built.
+
+    There is no fallback path: without the HIP library nothing in this package computes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise LibraryMissing(
+            "%s is missing: build it with `python -m motifcl_amd.build` "
+            "(or __graft_entry__.build())" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+class MccError(RuntimeError):
+    """Raised when a C-ABI call reports failure; carries mcc_last_error()."""
+
+    def __init__(self, code, message):
+        super().__init__("motifcl_amd error %d: %s" % (code, message))
+        self.code = code
+        self.message = message
+
+
+def check(rc):
+    if rc != 0:
+        raise MccError(rc, load().mcc_last_error().decode())

@@ -1,0 +1,95 @@
+"""Thin Python front of the C ABI.  torch is used only as the owner of device
+memory and of the current HIP stream; every computation happens in
+libmotifcl_amd.so."""
+import torch
+
+from . import lib as _lib
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream or None
+
+
+def _buf(t, dtype):
+    if not t.is_cuda:
+        raise ValueError("expected a device tensor")
+    if t.dtype != dtype:
+        raise ValueError("expected dtype %s, got %s" % (dtype, t.dtype))
+    if not t.is_contiguous():
+        raise ValueError("expected a contiguous tensor")
+    return t.data_ptr(), t.numel() * t.element_size()
+
+
+def apply_update_dense(state, scale, v, grad_w, C, lr, lr_scale, rms_beta, rms_eps, seed,
+                       in_features=None, out_features=None):
+    """In-place update-only step (CounterStateLinear::apply_update_seed)."""
+    L = _lib.load()
+    if in_features is None:
+        out_features, in_features = grad_w.shape
+    _lib.check(L.mcc_compact_counter_apply_update_dense(
+        _stream(), *_buf(state, torch.uint8), *_buf(scale, torch.float32), *_buf(v, torch.float32),
+        *_buf(grad_w, torch.float32), C, in_features, out_features,
+        lr, lr_scale, rms_beta, rms_eps, seed & 0xFFFFFFFF))
+
+
+def fused_workspace_nbytes(in_features, out_features, batch):
+    return int(_lib.load().mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch))
+
+
+def apply_update_fused(state, scale, v, grad_out, x, workspace, C, lr, lr_scale, rms_beta, rms_eps,
+                       seed):
+    """In-place fused step (CounterStateLinear::apply_update_backward)."""
+    L = _lib.load()
+    batch, out_features = grad_out.shape
+    in_features = x.shape[1]
+    if x.shape[0] != batch:
+        raise ValueError("x and grad_out disagree on the batch size")
+    _lib.check(L.mcc_compact_counter_apply_update_fused(
+        _stream(), *_buf(state, torch.uint8), *_buf(scale, torch.float32), *_buf(v, torch.float32),
+        *_buf(grad_out, torch.float32), *_buf(x, torch.float32),
+        workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+        C, in_features, out_features, batch, lr, lr_scale, rms_beta, rms_eps, seed & 0xFFFFFFFF))
+
+
+def matmul_transpose_a(a, b, out=None):
+    """c[m,n] = a[k,m]^T . b[k,n]."""
+    L = _lib.load()
+    k, m = a.shape
+    k2, n = b.shape
+    if k != k2:
+        raise ValueError("matmul_transpose_a: leading dimensions differ")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _lib.check(L.mcc_matmul_transpose_a_f32(_stream(), *_buf(a, torch.float32), *_buf(b, torch.float32),
+                                            *_buf(out, torch.float32), k, m, n))
+    return out
+
+
+def decode_weight(state, scale, C, in_features, out_features):
+    L = _lib.load()
+    w = torch.empty((out_features, in_features), dtype=torch.float32, device=state.device)
+    _lib.check(L.mcc_compact_counter_decode_weight(
+        _stream(), *_buf(state, torch.uint8), *_buf(scale, torch.float32), *_buf(w, torch.float32),
+        in_features, out_features, C))
+    return w
+
+
+def forward(x, state, scale, C, out_features):
+    L = _lib.load()
+    batch, in_features = x.shape
+    y = torch.empty((batch, out_features), dtype=torch.float32, device=x.device)
+    _lib.check(L.mcc_compact_counter_forward_u8(
+        _stream(), *_buf(x, torch.float32), *_buf(state, torch.uint8), *_buf(scale, torch.float32),
+        *_buf(y, torch.float32), batch, in_features, out_features, C))
+    return y
+
+
+def backward_input(grad_out, state, scale, C, in_features):
+    L = _lib.load()
+    batch, out_features = grad_out.shape
+    gx = torch.empty((batch, in_features), dtype=torch.float32, device=grad_out.device)
+    _lib.check(L.mcc_compact_counter_backward_input_u8(
+        _stream(), *_buf(state, torch.uint8), *_buf(scale, torch.float32),
+        *_buf(grad_out, torch.float32), *_buf(gx, torch.float32),
+        batch, in_features, out_features, C))
+    return gx
