@@ -1,0 +1,276 @@
+#!/usr/bin/env python3
+"""Benchmark of the compact-counter update on one MI355X.
+
+Primary line (BASELINE config 4): the fused step of one 7B-shaped layer -- seven counter
+tensors, 32768 tokens -- through mcc_compact_counter_apply_update_fused.  A "step" is one
+fused update of all seven tensors.  The same JSON line carries, under "update_only",
+BASELINE config 3: the update-only step over 224 7B-shaped tensors with precomputed
+gradients (6.476 G counters, 25.9 GB of gradient, distinct buffer per tensor).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg0|cfg1|cfg2|cfg4]
+                    [--no-update-only] [--no-cpu]
+
+Inputs are synthetic and seeded (torch generator, seed 0): X ~ N(0,1), dY ~ N(0,0.01),
+G ~ N(0,0.01), codes uniform on [0,62], scale = sqrt(3/(2 in)), v = 0, C = 11, lr = 3e-3,
+lr_scale = 0, rms_beta = 0.9, rms_eps = 1e-3.  Everything is resident in HBM before the
+timed region.  Kernel durations for the roofline come from HIP events recorded by the
+library on the launch stream inside the timed region.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_F32_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+C, LR, LR_SCALE, BETA, EPS = 11, 3e-3, 0.0, 0.9, 1e-3
+BYTES_PER_PARAM = 5.5          # 4 (read G) + 0.75 (read state) + 0.75 (write state)
+
+
+def layer_shapes(dim, hidden):
+    """(out, in) of the seven linears of one block: Wq Wk Wv Wo, W1 W3, W2."""
+    return [(dim, dim)] * 4 + [(hidden, dim)] * 2 + [(dim, hidden)]
+
+
+WORKLOADS = {
+    # name: (description, [(out,in)...] per layer, layers, tokens)
+    "cfg0": ("cfg0: single 288x288 counter linear, 4096 tokens, one fused update", [(288, 288)], 1, 4096),
+    "cfg1": ("cfg1: stories15M-shaped full step (dim 288, hidden 768, 6 layers = 42 tensors), 8192 tokens",
+             layer_shapes(288, 768), 6, 8192),
+    "cfg2": ("cfg2: 110M-shaped step (dim 768, hidden 2048, 12 layers = 84 tensors), 16384 tokens",
+             layer_shapes(768, 2048), 12, 16384),
+    "cfg4": ("cfg4: 7B-shaped single-layer fused step (d=4096, hidden 11008, 7 linears), 32768 tokens",
+             layer_shapes(4096, 11008), 1, 32768),
+}
+
+
+def pack_codes_torch(codes):
+    """[out, in] uint8 codes -> packed state bytes, 4 codes per 3 bytes (little-endian word)."""
+    import torch
+    c = codes.view(-1, 4).to(torch.int32)
+    w = c[:, 0] | (c[:, 1] << 6) | (c[:, 2] << 12) | (c[:, 3] << 18)
+    b = torch.stack([w & 0xFF, (w >> 8) & 0xFF, (w >> 16) & 0xFF], dim=1)
+    return b.to(torch.uint8).reshape(-1).contiguous()
+
+
+def make_state(gen, n_out, n_in):
+    import torch
+    codes = torch.randint(0, 63, (n_out, n_in), dtype=torch.uint8, device="cuda", generator=gen)
+    state = pack_codes_torch(codes)
+    scale = torch.full((n_out,), math.sqrt(3.0 / (2.0 * n_in)), dtype=torch.float32, device="cuda")
+    v = torch.zeros(n_out, dtype=torch.float32, device="cuda")
+    return state, scale, v
+
+
+def query(L, name):
+    import ctypes
+    ms, n = ctypes.c_double(), ctypes.c_uint64()
+    rc = L.mcc_profiler_query(name.encode(), ctypes.byref(ms), ctypes.byref(n))
+    assert rc == 0, L.mcc_last_error()
+    return ms.value, n.value
+
+
+def time_steps(step_fn, steps, warmup):
+    import torch
+    for i in range(warmup):
+        step_fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step_fn(warmup + i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def bench_fused(L, ops, name, steps, warmup):
+    import torch
+    desc, shapes, layers, tokens = WORKLOADS[name]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    tensors = []
+    ws_bytes = 0
+    xs, dys = {}, {}
+    for layer in range(layers):
+        for (n_out, n_in) in shapes:
+            # activations are shared by width inside a layer stack to bound memory on the small
+            # configs; each 7B tensor still streams its own X/dY rows from HBM (>= 537 MB each)
+            if n_in not in xs:
+                xs[n_in] = torch.randn(tokens, n_in, device="cuda", generator=gen)
+            if n_out not in dys:
+                dys[n_out] = torch.randn(tokens, n_out, device="cuda", generator=gen) * 0.01
+            tensors.append((make_state(gen, n_out, n_in), dys[n_out], xs[n_in], n_out, n_in))
+            ws_bytes = max(ws_bytes, ops.fused_workspace_nbytes(n_in, n_out, tokens))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    params = sum(t[3] * t[4] for t in tensors)
+    flops = sum(2.0 * tokens * t[3] * t[4] for t in tensors)
+
+    def step(i):
+        for k, ((state, scale, v), dy, x, n_out, n_in) in enumerate(tensors):
+            ops.apply_update_fused(state, scale, v, dy, x, ws, C, LR, LR_SCALE, BETA, EPS,
+                                   12345 + k + 1000 * i)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    L.mcc_profiler_reset()
+    L.mcc_profiler_enable(1)
+    ms_per_step = time_steps(step, steps, 0)
+    gemm_ms, gemm_n = query(L, "gemm_tn_f32")
+    upd_ms, upd_n = query(L, "counter_update")
+    L.mcc_profiler_enable(0)
+    L.mcc_profiler_reset()
+    # dominant kernel: the contraction.  One launch per tensor; flops per launch differ by
+    # tensor, so achieved = (total algorithmic flops of the launches) / (their total duration).
+    achieved = flops * steps / (gemm_ms * 1e-3) / 1e12
+    out = {
+        "value": params / (ms_per_step * 1e-3) / 1e9,
+        "ms_per_step": ms_per_step,
+        "config": {"workload": desc, "tensors": len(tensors), "params": params, "tokens": tokens,
+                   "C": C, "lr": LR, "lr_scale": LR_SCALE, "rms_beta": BETA, "rms_eps": EPS},
+        "roofline": {"bound": "mfma", "kernel": "gemm_tn_f32", "achieved": achieved,
+                     "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_MFMA_F32_TFLOPS, "traffic": None,
+                     "launches": gemm_n, "avg_launch_ms": gemm_ms / max(gemm_n, 1),
+                     "algorithmic_flops_per_step": flops},
+        "kernel_ms_per_step": {"gemm_tn_f32": gemm_ms / steps, "counter_update": upd_ms / steps},
+    }
+    sample = tensors[0]
+    del ws
+    return out, sample, tokens
+
+
+def bench_update_only(L, ops, steps, warmup):
+    import torch
+    shapes = layer_shapes(4096, 11008)
+    layers = 32
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    tensors = []
+    for layer in range(layers):
+        for (n_out, n_in) in shapes:
+            g = torch.randn(n_out, n_in, device="cuda", generator=gen) * 0.01
+            tensors.append((make_state(gen, n_out, n_in), g, n_out, n_in))
+    params = sum(t[2] * t[3] for t in tensors)
+
+    def step(i):
+        for k, ((state, scale, v), g, n_out, n_in) in enumerate(tensors):
+            ops.apply_update_dense(state, scale, v, g, C, LR, LR_SCALE, BETA, EPS, 12345 + k + 1000 * i)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    L.mcc_profiler_reset()
+    L.mcc_profiler_enable(1)
+    ms_per_step = time_steps(step, steps, 0)
+    upd_ms, upd_n = query(L, "counter_update")
+    L.mcc_profiler_enable(0)
+    L.mcc_profiler_reset()
+    achieved = BYTES_PER_PARAM * params * steps / (upd_ms * 1e-3) / 1e9
+    out = {
+        "metric": "counter-synapse updates/s (Gparam/s), update-only",
+        "value": params / (ms_per_step * 1e-3) / 1e9, "unit": "Gparam/s",
+        "ms_per_step": ms_per_step, "steps": steps, "warmup": warmup,
+        "config": {"workload": "cfg3: update-only, 224 7B-shaped tensors (32 layers x 7), "
+                               "precomputed fp32 G, distinct buffer per tensor",
+                   "tensors": len(tensors), "params": params},
+        "roofline": {"bound": "hbm", "kernel": "update_rows_kernel", "achieved": achieved,
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
+                     "traffic": None, "launches": upd_n, "avg_launch_ms": upd_ms / max(upd_n, 1),
+                     "algorithmic_bytes_per_param": BYTES_PER_PARAM},
+    }
+    sample = tensors[0]
+    return out, sample
+
+
+def cpu_baseline_fused(sample, tokens, rows, min_seconds=8.0):
+    """Times the CPU oracle's fused update on the first `rows` rows of one tensor."""
+    import numpy as np
+    from oracle import counter_oracle as oracle
+    (state, scale, v), dy, x, n_out, n_in = sample
+    rows = min(rows, n_out)
+    rb = n_in // 4 * 3
+    h_state = state[: rows * rb].cpu().numpy().copy()
+    h_scale, h_v = scale[:rows].cpu().numpy().copy(), v[:rows].cpu().numpy().copy()
+    h_dy = np.ascontiguousarray(dy[:, :rows].cpu().numpy())
+    h_x = x.cpu().numpy()
+    t0 = time.perf_counter()
+    passes = 0
+    while passes == 0 or time.perf_counter() - t0 < min_seconds:
+        oracle.update_fused(h_state, h_scale, h_v, h_dy, h_x, C, LR, LR_SCALE, BETA, EPS, 12345 + passes)
+        passes += 1
+    dt = time.perf_counter() - t0
+    return {"value": passes * rows * n_in / dt / 1e9, "unit": "Gparam/s", "cores": oracle.num_threads(),
+            "kind": "port", "seconds": dt,
+            "sample": "CPU oracle (C, -O3 -mavx2 -ffp-contract=off, OpenMP) fused update of the first %d "
+                      "rows of one [%d,%d] tensor at %d tokens (%.0f GFLOP per pass), %d passes; "
+                      "extrapolates linearly in rows"
+                      % (rows, n_out, n_in, tokens, 2.0 * tokens * rows * n_in / 1e9, passes)}
+
+
+def cpu_baseline_dense(sample, min_seconds=4.0):
+    from oracle import counter_oracle as oracle
+    (state, scale, v), g, n_out, n_in = sample
+    h = [t.cpu().numpy().copy() for t in (state, scale, v, g)]
+    t0 = time.perf_counter()
+    reps = 0
+    while reps == 0 or time.perf_counter() - t0 < min_seconds:
+        oracle.update_dense(h[0], h[1], h[2], h[3], C, LR, LR_SCALE, BETA, EPS, 12345 + reps)
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": reps * n_out * n_in / dt / 1e9, "unit": "Gparam/s", "cores": oracle.num_threads(),
+            "kind": "port", "seconds": dt,
+            "sample": "CPU oracle update-only on one [%d,%d] tensor, %d passes" % (n_out, n_in, reps)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-update-only", action="store_true", help="skip the cfg3 update-only leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of one tensor for the CPU fused sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path shards by output row with no "
+                 "exchange); run with --gpus 1")
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: launched with WORLD_SIZE > 1; this build measures one GPU only")
+
+    import torch
+    import motifcl_amd
+    from motifcl_amd import ops
+    L = motifcl_amd.load()  # raises if the HIP library is missing: there is no fallback
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup)
+    line = {
+        "metric": "counter-synapse updates/s (Gparam/s)",
+        "value": fused["value"], "unit": "Gparam/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": fused["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": fused["config"], "roofline": fused["roofline"],
+        "kernel_ms_per_step": fused["kernel_ms_per_step"],
+        "device": L.mcc_device_name().decode(),
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_fused(fused_sample, tokens, args.cpu_rows)
+    del fused_sample
+    torch.cuda.empty_cache()
+    if not args.no_update_only:
+        uo, uo_sample = bench_update_only(L, ops, args.steps, args.warmup)
+        if not args.no_cpu:
+            uo["cpu_baseline"] = cpu_baseline_dense(uo_sample)
+        line["update_only"] = uo
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -163,6 +163,19 @@ int mcc_memset_zero(void* stream, void* dst, size_t nbytes);
  * src/runtime/backend.cpp:328-331). */
 int mcc_stream_synchronize(void* stream);
 
+/*
+ * Per-kernel GPU timing.  While enabled, each kernel launched through this ABI is
+ * bracketed by HIP events on its launch stream; mcc_profiler_query waits for them and
+ * returns the summed duration and launch count of one kernel family:
+ * "gemm_tn_f32", "counter_update", "counter_decode_weight", "counter_forward",
+ * "counter_backward_input".  Replaces Profiler (src/runtime/profiler.cpp) and
+ * VulkanRuntime::set_gpu_timing_enabled / last_gpu_time_us
+ * (include/motifcl/runtime/vulkan_backend.hpp:181-185).
+ */
+void mcc_profiler_enable(int on);
+void mcc_profiler_reset(void);
+int mcc_profiler_query(const char* kernel_name, double* total_ms, uint64_t* launches);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,60 @@ void track_alloc(size_t n) {
     }
 }
 
+// ---- per-kernel GPU timing ---------------------------------------------------
+// When enabled, every kernel launch made through this ABI is bracketed by two HIP
+// events on the launch stream (the reference's counterpart: Profiler /
+// VulkanRuntime::set_gpu_timing_enabled, include/motifcl/runtime/vulkan_backend.hpp:181-185).
+struct TimedLaunch {
+    const char* name;
+    hipEvent_t start, stop;
+};
+struct Profiler {
+    std::mutex mu;
+    bool enabled = false;
+    std::vector<TimedLaunch> records;
+    std::vector<hipEvent_t> spare;
+    hipEvent_t take() {
+        if (!spare.empty()) {
+            hipEvent_t e = spare.back();
+            spare.pop_back();
+            return e;
+        }
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) return nullptr;
+        return e;
+    }
+};
+Profiler& profiler() {
+    static Profiler p;
+    return p;
+}
+
+class ScopedKernelTimer {
+public:
+    ScopedKernelTimer(const char* name, hipStream_t stream) : stream_(stream) {
+        Profiler& p = profiler();
+        std::lock_guard<std::mutex> lock(p.mu);
+        if (!p.enabled) return;
+        rec_.name = name;
+        rec_.start = p.take();
+        rec_.stop = p.take();
+        active_ = rec_.start && rec_.stop;
+        if (active_) (void)hipEventRecord(rec_.start, stream_);
+    }
+    ~ScopedKernelTimer() {
+        if (!active_) return;
+        (void)hipEventRecord(rec_.stop, stream_);
+        Profiler& p = profiler();
+        std::lock_guard<std::mutex> lock(p.mu);
+        p.records.push_back(rec_);
+    }
+private:
+    hipStream_t stream_;
+    TimedLaunch rec_{};
+    bool active_ = false;
+};
+
 }  // namespace
 
 extern "C" {
@@ -129,9 +183,12 @@ int mcc_compact_counter_apply_update_dense(void* stream, uint8_t* state, size_t 
     if (reinterpret_cast<uintptr_t>(grad_w) % alignof(float) || reinterpret_cast<uintptr_t>(scale) % alignof(float) ||
         reinterpret_cast<uintptr_t>(v) % alignof(float))
         return fail(MCC_E_INVALID, "compact-counter update float buffers must be 4-byte aligned");
-    const hipError_t e = mcc::launch_update_dense(static_cast<hipStream_t>(stream), state, scale, v, grad_w,
-                                                  (int)C, (int)in_features, (int)out_features, lr,
-                                                  lr_scale, rms_beta, rms_eps, seed);
+    hipError_t e;
+    {
+        ScopedKernelTimer timer("counter_update", static_cast<hipStream_t>(stream));
+        e = mcc::launch_update_dense(static_cast<hipStream_t>(stream), state, scale, v, grad_w, (int)C,
+                                     (int)in_features, (int)out_features, lr, lr_scale, rms_beta, rms_eps, seed);
+    }
     if (e != hipSuccess) return hip_fail(e, "compact-counter update launch failed");
     return MCC_OK;
 }
@@ -180,10 +237,17 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
         return fail(MCC_E_INVALID, "compact-counter fused update float buffers must be 4-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* grad_w = static_cast<float*>(workspace);
-    hipError_t e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features);
+    hipError_t e;
+    {
+        ScopedKernelTimer timer("gemm_tn_f32", s);
+        e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features);
+    }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
-    e = mcc::launch_update_dense(s, state, scale, v, grad_w, (int)C, (int)in_features, (int)out_features, lr,
-                                 lr_scale, rms_beta, rms_eps, seed);
+    {
+        ScopedKernelTimer timer("counter_update", s);
+        e = mcc::launch_update_dense(s, state, scale, v, grad_w, (int)C, (int)in_features, (int)out_features, lr,
+                                     lr_scale, rms_beta, rms_eps, seed);
+    }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update launch failed");
     return MCC_OK;
 }
@@ -204,7 +268,11 @@ int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, co
     if (reinterpret_cast<uintptr_t>(a) % alignof(float) || reinterpret_cast<uintptr_t>(b) % alignof(float) ||
         reinterpret_cast<uintptr_t>(c) % alignof(float))
         return fail(MCC_E_INVALID, "matmul_transpose_a buffers must be 4-byte aligned");
-    const hipError_t e = mcc::launch_gemm_tn_f32(static_cast<hipStream_t>(stream), a, b, c, (int)k, (int)m, (int)n);
+    hipError_t e;
+    {
+        ScopedKernelTimer timer("gemm_tn_f32", static_cast<hipStream_t>(stream));
+        e = mcc::launch_gemm_tn_f32(static_cast<hipStream_t>(stream), a, b, c, (int)k, (int)m, (int)n);
+    }
     if (e != hipSuccess) return hip_fail(e, "matmul_transpose_a launch failed");
     return MCC_OK;
 }
@@ -220,6 +288,7 @@ int mcc_compact_counter_decode_weight(void* stream, const uint8_t* state, size_t
     if (scale_nbytes < out_features * sizeof(float)) return fail(MCC_E_INVALID, "compact-counter scale buffer is too small");
     if (weight_nbytes < out_features * in_features * sizeof(float))
         return fail(MCC_E_INVALID, "compact-counter weight buffer is too small");
+    ScopedKernelTimer timer("counter_decode_weight", static_cast<hipStream_t>(stream));
     const hipError_t e = mcc::launch_decode_weight(static_cast<hipStream_t>(stream), state, scale, weight, (int)C,
                                                    (int)in_features, (int)out_features);
     if (e != hipSuccess) return hip_fail(e, "compact-counter decode launch failed");
@@ -243,6 +312,7 @@ int mcc_compact_counter_forward_u8(void* stream, const float* x, size_t x_nbytes
         return fail(MCC_E_INVALID, "compact-counter forward buffer size overflows size_t");
     if (x_nbytes < batch * in_features * sizeof(float) || out_nbytes < batch * out_features * sizeof(float))
         return fail(MCC_E_INVALID, "compact-counter forward activation buffer is too small");
+    ScopedKernelTimer timer("counter_forward", static_cast<hipStream_t>(stream));
     const hipError_t e = mcc::launch_forward(static_cast<hipStream_t>(stream), x, state, scale, out, (int)C,
                                              (int)batch, (int)in_features, (int)out_features);
     if (e != hipSuccess) return hip_fail(e, "compact-counter forward launch failed");
@@ -269,6 +339,7 @@ int mcc_compact_counter_backward_input_u8(void* stream, const uint8_t* state, si
         return fail(MCC_E_INVALID, "compact-counter grad_out buffer is too small");
     if (grad_x_nbytes < batch * in_features * sizeof(float))
         return fail(MCC_E_INVALID, "compact-counter grad_x buffer is too small");
+    ScopedKernelTimer timer("counter_backward_input", static_cast<hipStream_t>(stream));
     const hipError_t e = mcc::launch_backward_input(static_cast<hipStream_t>(stream), grad_out, state, scale,
                                                     grad_x, (int)C, (int)batch, (int)in_features,
                                                     (int)out_features);
@@ -382,6 +453,42 @@ int mcc_memset_zero(void* stream, void* dst, size_t nbytes) {
                        static_cast<uint8_t*>(dst), nbytes);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e, "device memset failed");
+    return MCC_OK;
+}
+
+void mcc_profiler_enable(int on) {
+    Profiler& p = profiler();
+    std::lock_guard<std::mutex> lock(p.mu);
+    p.enabled = on != 0;
+}
+
+void mcc_profiler_reset(void) {
+    Profiler& p = profiler();
+    std::lock_guard<std::mutex> lock(p.mu);
+    for (const TimedLaunch& r : p.records) {
+        p.spare.push_back(r.start);
+        p.spare.push_back(r.stop);
+    }
+    p.records.clear();
+}
+
+int mcc_profiler_query(const char* kernel_name, double* total_ms, uint64_t* launches) {
+    if (!kernel_name || !total_ms || !launches) return fail(MCC_E_INVALID, "profiler query received a null pointer");
+    Profiler& p = profiler();
+    std::lock_guard<std::mutex> lock(p.mu);
+    double sum = 0.0;
+    uint64_t n = 0;
+    for (const TimedLaunch& r : p.records) {
+        if (std::string(r.name) != kernel_name) continue;
+        hipError_t e = hipEventSynchronize(r.stop);
+        float ms = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, r.start, r.stop);
+        if (e != hipSuccess) return hip_fail(e, "profiler query failed");
+        sum += ms;
+        ++n;
+    }
+    *total_ms = sum;
+    *launches = n;
     return MCC_OK;
 }
 

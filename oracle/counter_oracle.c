@@ -259,23 +259,32 @@ int oracle_update_dense(uint8_t *state, float *scale, float *v, const float *gra
 
 /* ---- weight gradient, sequential in r: kernels/compact_counter.cl:174-175 - */
 /* gw[o,i] = (((0 + dY[0,o]*X[0,i]) + dY[1,o]*X[1,i]) + ...), fp32.  The loop
- * nest puts r outside a block of rows so the per-element order over r is
- * unchanged while X rows stream through cache.                               */
+ * nest blocks rows and columns so that X streams through cache once per block
+ * of 8 rows; every element still accumulates r = 0..N-1 in order.            */
 void oracle_grad_w_seq(const float *grad_out, const float *x, float *grad_w,
                        int in_features, int out_features, int N) {
-#pragma omp parallel for schedule(static)
-    for (int o = 0; o < out_features; ++o) {
-        float *g_row = grad_w + (size_t)o * in_features;
-        for (int i = 0; i < in_features; ++i) g_row[i] = 0.0f;
-        for (int r = 0; r < N; ++r) {
-            float go = grad_out[(size_t)r * out_features + o];
-            const float *x_row = x + (size_t)r * in_features;
-            for (int i = 0; i < in_features; ++i) {
-                float p = go * x_row[i];
-                g_row[i] = g_row[i] + p;
+    enum { OB = 8, IB = 1024 }; /* rows and columns per block: 32 KiB of accumulators */
+    int n_ob = (out_features + OB - 1) / OB;
+    int n_ib = (in_features + IB - 1) / IB;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int ob = 0; ob < n_ob; ++ob)
+        for (int ib = 0; ib < n_ib; ++ib) {
+            int o0 = ob * OB, o1 = o0 + OB < out_features ? o0 + OB : out_features;
+            int i0 = ib * IB, i1 = i0 + IB < in_features ? i0 + IB : in_features;
+            for (int o = o0; o < o1; ++o)
+                for (int i = i0; i < i1; ++i) grad_w[(size_t)o * in_features + i] = 0.0f;
+            for (int r = 0; r < N; ++r) {
+                const float *x_row = x + (size_t)r * in_features;
+                for (int o = o0; o < o1; ++o) {
+                    float go = grad_out[(size_t)r * out_features + o];
+                    float *g_row = grad_w + (size_t)o * in_features;
+                    for (int i = i0; i < i1; ++i) {
+                        float p = go * x_row[i];
+                        g_row[i] = g_row[i] + p;
+                    }
+                }
             }
         }
-    }
 }
 
 /* ---- fused update: src/nn/compact_counter.cpp:158-231 --------------------- */
