@@ -58,6 +58,31 @@ int mcc_compact_counter_apply_update_dense(
     float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
 
 /*
+ * Update-only step for a list of counter tensors in one call -- the optimizer step of a
+ * whole model when every dense weight gradient is already in memory.  Each tensor gets
+ * exactly the result of mcc_compact_counter_apply_update_dense with its own lr and seed;
+ * C, lr_scale, rms_beta and rms_eps are shared.  The reference applies the update layer by
+ * layer from the host (CounterStateLinear::apply_update_seed,
+ * src/nn/compact_counter.cpp:113-156, once per module; the layer lists it walks are e.g.
+ * tools/train_ternary15m.cpp:313-318); one launch over the rows of many tensors keeps the
+ * memory system and the ALUs busy together, which a single small tensor cannot.
+ * `tensors` is a host array; tensors must not alias each other.
+ */
+typedef struct mcc_counter_tensor {
+    uint8_t* state;      size_t state_nbytes;
+    float* scale;        size_t scale_nbytes;
+    float* v;            size_t v_nbytes;
+    const float* grad_w; size_t grad_w_nbytes;
+    size_t in_features, out_features;
+    float lr;
+    uint32_t seed;
+} mcc_counter_tensor;
+
+int mcc_compact_counter_apply_update_dense_batched(
+    void* stream, const mcc_counter_tensor* tensors, size_t n_tensors,
+    size_t C, float lr_scale, float rms_beta, float rms_eps);
+
+/*
  * Bytes of transient workspace mcc_compact_counter_apply_update_fused needs
  * for the given shape (0 on invalid dimensions).
  */

@@ -160,34 +160,62 @@ const char* mcc_device_name(void) {
     return name.c_str();
 }
 
+// Validation shared by the single and the batched update-only entry points; fills `out`.
+static int check_update_tensor(const mcc_counter_tensor& t, size_t C, float lr_scale, float rms_beta,
+                               float rms_eps, mcc::UpdateTensor* out) {
+    const char* what = "compact-counter update";
+    if (!check_codec(what, C, t.in_features, t.out_features)) return MCC_E_INVALID;
+    if (!std::isfinite(t.lr)) return fail(MCC_E_INVALID, "compact-counter update requires finite lr");
+    if (!std::isfinite(lr_scale)) return fail(MCC_E_INVALID, "compact-counter update requires finite lr_scale");
+    if (!std::isfinite(rms_beta)) return fail(MCC_E_INVALID, "compact-counter update requires finite rms_beta");
+    if (!std::isfinite(rms_eps) || rms_eps < 0.0f)
+        return fail(MCC_E_INVALID, "compact-counter update requires non-negative finite rms_eps");
+    if (!t.state || !t.scale || !t.v || !t.grad_w)
+        return fail(MCC_E_INVALID, "compact-counter update received a null buffer");
+    const size_t n_groups = t.out_features * (t.in_features / 4);
+    if (t.state_nbytes < n_groups * 3) return fail(MCC_E_INVALID, "compact-counter update state buffer is too small");
+    if (t.scale_nbytes < t.out_features * sizeof(float) || t.v_nbytes < t.out_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter update per-row buffer is too small");
+    if (t.grad_w_nbytes < t.out_features * t.in_features * sizeof(float))
+        return fail(MCC_E_INVALID, "compact-counter update gradient buffer is too small");
+    if (reinterpret_cast<uintptr_t>(t.grad_w) % alignof(float) || reinterpret_cast<uintptr_t>(t.scale) % alignof(float) ||
+        reinterpret_cast<uintptr_t>(t.v) % alignof(float))
+        return fail(MCC_E_INVALID, "compact-counter update float buffers must be 4-byte aligned");
+    out->state = t.state; out->scale = t.scale; out->v = t.v; out->grad_w = t.grad_w;
+    out->in_features = (int)t.in_features; out->out_features = (int)t.out_features;
+    out->row_start = 0; out->seed = t.seed; out->lr = t.lr; out->pad = 0;
+    return MCC_OK;
+}
+
 int mcc_compact_counter_apply_update_dense(void* stream, uint8_t* state, size_t state_nbytes,
                                            float* scale, size_t scale_nbytes, float* v,
                                            size_t v_nbytes, const float* grad_w,
                                            size_t grad_w_nbytes, size_t C, size_t in_features,
                                            size_t out_features, float lr, float lr_scale,
                                            float rms_beta, float rms_eps, uint32_t seed) {
-    const char* what = "compact-counter update";
-    if (!check_codec(what, C, in_features, out_features)) return MCC_E_INVALID;
-    if (!std::isfinite(lr)) return fail(MCC_E_INVALID, "compact-counter update requires finite lr");
-    if (!std::isfinite(lr_scale)) return fail(MCC_E_INVALID, "compact-counter update requires finite lr_scale");
-    if (!std::isfinite(rms_beta)) return fail(MCC_E_INVALID, "compact-counter update requires finite rms_beta");
-    if (!std::isfinite(rms_eps) || rms_eps < 0.0f)
-        return fail(MCC_E_INVALID, "compact-counter update requires non-negative finite rms_eps");
-    if (!state || !scale || !v || !grad_w) return fail(MCC_E_INVALID, "compact-counter update received a null buffer");
-    const size_t n_groups = out_features * (in_features / 4);
-    if (state_nbytes < n_groups * 3) return fail(MCC_E_INVALID, "compact-counter update state buffer is too small");
-    if (scale_nbytes < out_features * sizeof(float) || v_nbytes < out_features * sizeof(float))
-        return fail(MCC_E_INVALID, "compact-counter update per-row buffer is too small");
-    if (grad_w_nbytes < out_features * in_features * sizeof(float))
-        return fail(MCC_E_INVALID, "compact-counter update gradient buffer is too small");
-    if (reinterpret_cast<uintptr_t>(grad_w) % alignof(float) || reinterpret_cast<uintptr_t>(scale) % alignof(float) ||
-        reinterpret_cast<uintptr_t>(v) % alignof(float))
-        return fail(MCC_E_INVALID, "compact-counter update float buffers must be 4-byte aligned");
+    const mcc_counter_tensor t = {state, state_nbytes, scale, scale_nbytes, v, v_nbytes, grad_w, grad_w_nbytes,
+                                  in_features, out_features, lr, seed};
+    return mcc_compact_counter_apply_update_dense_batched(stream, &t, 1, C, lr_scale, rms_beta, rms_eps);
+}
+
+int mcc_compact_counter_apply_update_dense_batched(void* stream, const mcc_counter_tensor* tensors,
+                                                   size_t n_tensors, size_t C, float lr_scale,
+                                                   float rms_beta, float rms_eps) {
+    if (n_tensors == 0) return MCC_OK;
+    if (!tensors) return fail(MCC_E_INVALID, "compact-counter update received a null tensor list");
+    std::vector<mcc::UpdateTensor> dev(n_tensors);
+    for (size_t i = 0; i < n_tensors; ++i) {
+        const int rc = check_update_tensor(tensors[i], C, lr_scale, rms_beta, rms_eps, &dev[i]);
+        if (rc != MCC_OK) {
+            if (n_tensors > 1) g_error = "tensor " + std::to_string(i) + ": " + g_error;
+            return rc;
+        }
+    }
     hipError_t e;
     {
         ScopedKernelTimer timer("counter_update", static_cast<hipStream_t>(stream));
-        e = mcc::launch_update_dense(static_cast<hipStream_t>(stream), state, scale, v, grad_w, (int)C,
-                                     (int)in_features, (int)out_features, lr, lr_scale, rms_beta, rms_eps, seed);
+        e = mcc::launch_update_batch(static_cast<hipStream_t>(stream), dev.data(), n_tensors, (int)C, lr_scale,
+                                     rms_beta, rms_eps);
     }
     if (e != hipSuccess) return hip_fail(e, "compact-counter update launch failed");
     return MCC_OK;

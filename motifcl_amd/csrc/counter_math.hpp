@@ -33,16 +33,6 @@ MCC_HD uint32_t hash_u32(uint32_t x) {
 // 24-bit word of one packed group -> code k (kernels/compact_counter.cl:25-31)
 MCC_HD uint32_t code_of(uint32_t word, int k) { return (word >> (6 * k)) & 0x3fu; }
 
-// Per-row constants of the tick (kernels/compact_counter.cl:118,123-124): the
-// reference evaluates them per element from the same per-row operands, so
-// hoisting them changes no bit.
-struct RowConsts {
-    float dn;      // denom[row]
-    float k;       // Cf / s_new
-    float ratio;   // s_old / s_new
-    float neg_lr;  // -lr
-};
-
 // Constants of the state encoding for one counter depth C (lv = 2C-1 levels per
 // ternary value).  (code * magic) >> 16 == code / lv for every code < 64.
 struct Codec {
@@ -64,47 +54,151 @@ MCC_HD Codec make_codec(int C) {
 // t + 1 = code / lv  (kernels/compact_counter.cl:10)
 MCC_HD int code_q(uint32_t code, const Codec& cd) { return (int)((code * cd.magic) >> 16); }
 
-// Largest |floor(val)| that can still matter.  With t = code/lv - 1 in
-// [-1, 63/lv - 1] the ternary value saturates whenever |total| >= (63/lv + 1)*C,
-// which is <= 64 for every C with 3*(2C-1) <= 64; totals beyond that all give
-// the same saturated code, so floor(val) is clamped to +-kTotalClamp first.
-constexpr float kTotalClamp = 128.0f;
+// ---------------------------------------------------------------------------
+// The tick after val = c_reb + tick is a function of three small integers:
+// q = t + 1 (from the old code), total = floor(val) + [rnd < frac], and C
+// (kernels/compact_counter.cl:126-136).  It is tabulated once per kernel launch:
+//
+//   fin[(total + lim_neg) << shift | q] = new 6-bit code
+//
+// Range of `total` that can matter: with t = q - 1 in [-1, rows - 2]
+// (rows = 63/lv + 1 distinct q values) the ternary value saturates upward as
+// soon as carry >= 3, i.e. total >= 3C, and downward as soon as
+// carry <= -rows, i.e. total <= -rows*C.  floor(val) is therefore clamped to
+// [-lim_neg, lim_pos] = [-(rows*C + 1), 3C] first: every clamped value, with or
+// without the +1 of the stochastic round, lies in the same saturated region as
+// the unclamped one.  Valid for finite val (|val| < 2^31 in the reference's
+// own terms, where its float->int conversions stop being defined).
+// ---------------------------------------------------------------------------
+struct LutGeom {
+    int rows;      // distinct q = code / lv values
+    int shift;     // log2 of the q-stride of the table (power of two >= rows)
+    int lim_neg;   // clamp of floor(val) below, as a positive number
+    int lim_pos;   // clamp of floor(val) above
+    int width;     // number of distinct totals: lim_neg + lim_pos + 2
+};
+
+constexpr int kLutFinMaxBytes = 4480;  // C = 1: width 70 << shift 6
+
+MCC_HD LutGeom lut_geom(const Codec& cd) {
+    LutGeom g;
+    g.rows = 63 / cd.lv + 1;
+    g.shift = 0;
+    while ((1 << g.shift) < g.rows) ++g.shift;
+    g.lim_neg = g.rows * cd.C + 1;
+    g.lim_pos = 3 * cd.C;
+    g.width = g.lim_neg + g.lim_pos + 2;
+    return g;
+}
+
+// New code for old q = t + 1 and integer total = ccv (kernels/compact_counter.cl:129-136).
+MCC_HD uint32_t fin_entry(int total, int q, const Codec& cd) {
+    const int C = cd.C;
+    const int mag = total < 0 ? -total : total;
+    const int carry = total < 0 ? -(mag / C) : mag / C;  // trunc(ccv / Cf)
+    int rem = total - carry * C;                          // ccv - carry * Cf
+    const int nt = (q - 1) + carry;
+    const int ct = nt < -1 ? -1 : (nt > 1 ? 1 : nt);
+    if (ct != nt) rem = (total > 0 ? 1 : (total < 0 ? -1 : 0)) * (C - 1);
+    return (uint32_t)((ct + 1) * cd.lv + rem + (C - 1));
+}
+
+// Decode tables, indexed by the 6-bit code:
+//   q_off[code] = code / lv + (lim_neg << shift)   (t + 1, pre-biased for the fin index)
+//   c_reb[code] = (float)(code % lv - (C-1)) * (s_old / s_new)
+// c_reb is the rebased residual counter of kernels/compact_counter.cl:124; it depends on the
+// row through the scale ratio only, so it is tabulated once per row (64 products) instead of
+// once per weight.
+MCC_HD int code_c(uint32_t code, const Codec& cd) {
+    return (int)code - code_q(code, cd) * cd.lv - (cd.C - 1);
+}
+
+MCC_HD int q_off_entry(uint32_t code, const Codec& cd, const LutGeom& g) {
+    return code_q(code, cd) + (g.lim_neg << g.shift);
+}
+
+MCC_HD float c_reb_entry(uint32_t code, const Codec& cd, float ratio) {
+    return (float)code_c(code, cd) * ratio;
+}
+
+MCC_HD void fill_fin_entry(int idx, const Codec& cd, const LutGeom& g, uint8_t* fin) {
+    const int til = idx >> g.shift;
+    const int q = idx & ((1 << g.shift) - 1);
+    fin[idx] = q < g.rows ? (uint8_t)fin_entry(til - g.lim_neg, q, cd) : (uint8_t)0;
+}
+
+// Division by the per-row denominator, gw / dn, without a per-element reciprocal: with
+// r = RN(1/dn) computed once per row,
+//     q0 = RN(gw * r);  t = fma(-dn, q0, gw);  q1 = fma(t, r, q0);
+//     t  = fma(-dn, q1, gw);  q = fma(t, r, q1)
+// returns RN(gw / dn) exactly (Markstein: a faithful quotient corrected with the exact fma
+// residual and the correctly rounded reciprocal is the correctly rounded quotient), provided
+// no intermediate leaves the normal range.  That holds when dn is in [2^-40, 2^40] and every
+// gw of the row is zero or has |gw| in [2^-60, 2^50].  The row statistics pass collects what
+// the test needs: the sum of squares bounds |gw| from above, and the minimum over the row of
+// range_key(gw) bounds the non-zero |gw| from below.  Rows that fail take the plain division.
+MCC_HD uint32_t float_bits(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __float_as_uint(f);
+#else
+    uint32_t u;
+    __builtin_memcpy(&u, &f, 4);
+    return u;
+#endif
+}
+
+// Orders floats by magnitude with zero mapped above everything: (bits << 1) - 1.
+MCC_HD uint32_t range_key(float gw) { return (float_bits(gw) << 1) - 1u; }
+
+MCC_HD bool row_takes_fast_division(float dn, float row_sum_sq, uint32_t row_min_key) {
+    return dn >= 0x1p-40f && dn <= 0x1p40f && row_sum_sq < 0x1p100f && row_min_key >= range_key(0x1p-60f);
+}
+
+template <bool FAST>
+MCC_HD float div_by_row(float gw, float dn, float r) {
+    if (!FAST) return gw / dn;
+    float q = gw * r;
+    float t = fmaf(-dn, q, gw);
+    q = fmaf(t, r, q);
+    t = fmaf(-dn, q, gw);
+    q = fmaf(t, r, q);
+    return q;
+}
+
+MCC_HD float clamp_f(float x, float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_fmed3f(x, lo, hi);
+#else
+    return fminf(fmaxf(x, lo), hi);
+#endif
+}
+
+// Per-row constants of the tick (kernels/compact_counter.cl:118,123).
+struct TickConsts {
+    float dn, r;      // denom[row] and RN(1/denom[row])
+    float k;          // Cf / s_new
+    float neg_lr;     // -lr
+    float neg_lim_neg, lim_pos;  // clamp of floor(val), as floats
+    uint32_t seed;
+    int shift;
+};
 
 // One stochastic-rounding tick (kernels/compact_counter.cl:120-136).
-//   code  : current 6-bit code          gw   : weight gradient of this element
-//   elem  : row*in + i (the RNG index)  seed : update seed
+//   code : current 6-bit code           gw   : weight gradient of this element
+//   elem : row*in + i (the RNG index)
+//   c_reb, q_off : the decode tables above;  fin : the (total, q) -> code table
 // Returns the new 6-bit code.
-//
-// Differences in form (not in value) from the kernel text, valid for finite
-// inputs with |val| < 2^31:
-//  * floor(val) is clamped to +-kTotalClamp (see above);
-//  * carry = trunc(ccv / Cf) is evaluated as trunc((ccv +- 0.5) * (1/Cf)):
-//    ccv is an integer with |ccv| <= 129, so (|ccv| + 0.5)/C has a fractional
-//    part in [0.5/C, 1 - 0.5/C], at least 0.045 away from an integer, far more
-//    than the 2^-16 rounding error of the product;
-//  * rem = ccv - carry*Cf is one fma: both steps are exact on small integers.
-MCC_HD uint32_t tick_code(uint32_t code, float gw, const RowConsts& rc, uint32_t seed,
-                          uint32_t elem, const Codec& cd) {
-    const int C = cd.C, lv = cd.lv;
-    const float Cf = cd.Cf, inv_c = cd.inv_c;
-    const int q = code_q(code, cd);               // t + 1
-    const int c = (int)code - q * lv - (C - 1);
-    const float tick = (rc.neg_lr * (gw / rc.dn)) * rc.k;
-    const float c_reb = (float)c * rc.ratio;
-    const float val = c_reb + tick;
+template <bool FAST_DIV, typename CReb, typename QOff, typename Fin>
+MCC_HD uint32_t tick_code(uint32_t code, float gw, const TickConsts& tc, uint32_t elem,
+                          CReb c_reb, QOff q_off, Fin fin) {
+    const float tick = (tc.neg_lr * div_by_row<FAST_DIV>(gw, tc.dn, tc.r)) * tc.k;
+    const float val = c_reb[code] + tick;
     const float f = floorf(val);
     const float frac = val - f;
-    const uint32_t h = hash_u32(seed ^ hash_u32(elem));
+    const uint32_t h = hash_u32(tc.seed ^ hash_u32(elem));
     const float rnd = (float)(h & 0x00ffffffu) * (1.0f / 16777216.0f);
-    const float fc = fminf(fmaxf(f, -kTotalClamp), kTotalClamp);
-    const float ccv = fc + (rnd < frac ? 1.0f : 0.0f);
-    const float carry = truncf((ccv + copysignf(0.5f, ccv)) * inv_c);
-    float rem = fmaf(-carry, Cf, ccv);
-    const int nt = (q - 1) + (int)carry;
-    const int ct = nt < -1 ? -1 : (nt > 1 ? 1 : nt);
-    if (ct != nt) rem = fminf(fmaxf(ccv, -1.0f), 1.0f) * (Cf - 1.0f);
-    const int ri = (int)rem;
-    return (uint32_t)((ct + 1) * lv + ri + (C - 1));
+    const int til = (int)clamp_f(f, tc.neg_lim_neg, tc.lim_pos) + (rnd < frac ? 1 : 0);
+    return fin[((uint32_t)til << tc.shift) + (uint32_t)q_off[code]];
 }
 
 // Row statistics epilogue (kernels/compact_counter.cl:92-99), given the tree

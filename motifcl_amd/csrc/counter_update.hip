@@ -1,6 +1,6 @@
 // Update-only step of the compact-counter layer on gfx950: row statistics,
 // stochastic-rounding tick and scale commit in ONE kernel, one wave64 per
-// output row.
+// output row, for one tensor or a batch of tensors per launch.
 //
 // Why one wave per row: the reference's row reduction
 // (kernels/compact_counter.cl:75-91) is 64 strided partial sums (lane l walks
@@ -14,9 +14,17 @@
 // which needs the whole row's sum of squares first.  Holding the row (up to
 // 43 groups per lane for in = 11008) in VGPRs lets HBM see the gradient once:
 // 4 B (G) + 0.75 B (state read) + 0.75 B (state write) per weight.
+//
+// Why persistent waves over a batch: a wave alternates between waiting for its
+// row to arrive and ~45 VALU instructions per weight of tick arithmetic.  With
+// many more rows than resident waves the phases of different waves drift apart
+// and the memory system and the VALUs stay busy together; a single small
+// tensor is one synchronous round of load-then-compute.  The batched entry
+// point therefore walks the rows of up to 64 tensors in one launch.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <vector>
 
 #include "counter_math.hpp"
 #include "launch.hpp"
@@ -25,19 +33,34 @@ namespace mcc {
 namespace {
 
 constexpr int kWave = 64;
-constexpr int kWavesPerBlock = 4;
+constexpr int kWavesPerBlock = 1;  // one wave per workgroup: the row index is a function of blockIdx alone
+constexpr int kThreads = kWave * kWavesPerBlock;
 
-struct UpdateArgs {
-    uint8_t* state;
-    float* scale;
-    float* v;
-    const float* grad_w;
+struct BatchArgs {
+    UpdateTensor t[kMaxUpdateBatch];
+    int n_tensors;
+    int total_rows;
     Codec cd;
-    int in_features, out_features, gpr;
-    float lr, lr_scale, rms_beta, rms_eps;
-    uint32_t seed;
+    LutGeom geom;
+    float lr_scale, rms_beta, rms_eps;
 };
 
+// Per-workgroup tables in LDS (see counter_math.hpp).  fin and q_off depend on C only and are
+// built once per launch; c_reb depends on the row's scale ratio and is rebuilt per row.
+struct Luts {
+    uint8_t fin[kLutFinMaxBytes];
+    int q_off[64];
+    float c_reb[64];
+};
+
+__device__ __forceinline__ void build_luts(Luts& l, const Codec& cd, const LutGeom& geom) {
+    for (int i = threadIdx.x; i < 64; i += blockDim.x) l.q_off[i] = q_off_entry((uint32_t)i, cd, geom);
+    const int n = geom.width << geom.shift;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) fill_fin_entry(i, cd, geom, l.fin);
+    __syncthreads();
+}
+
+// Byte-granular access to one packed group (any alignment, any position).
 __device__ __forceinline__ uint32_t load_group(const uint8_t* p) {
     return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
 }
@@ -48,16 +71,34 @@ __device__ __forceinline__ void store_group(uint8_t* p, uint32_t w) {
     p[2] = (uint8_t)((w >> 16) & 0xffu);
 }
 
-__device__ __forceinline__ void accumulate(float& g_sq, float& grad_s, const float g[4], uint32_t w,
-                                           const Codec& cd, bool with_gs) {
+// One group's 24-bit word fetched with a single 4-byte load (global memory takes unaligned
+// dword accesses); the byte above the word belongs to the next group and is never looked
+// at.  The caller guarantees that byte exists, i.e. the group is not the tensor's last.
+__device__ __forceinline__ uint32_t load_group_dword(const uint8_t* p) {
+    uint32_t w;
+    __builtin_memcpy(&w, p, 4);
+    return w;
+}
+
+// Row statistics of one group (kernels/compact_counter.cl:78-83) plus the magnitude key
+// that decides whether the row may use the reciprocal-based division.
+struct RowAcc {
+    float g_sq = 0.0f, grad_s = 0.0f;
+    uint32_t min_key = 0xffffffffu;
+};
+
+template <bool WITH_GS>
+__device__ __forceinline__ void accumulate(RowAcc& acc, const float g[4], uint32_t w, const Codec& cd) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const float sq = g[k] * g[k];
-        g_sq = g_sq + sq;
-        if (with_gs) {
+        acc.g_sq = acc.g_sq + sq;
+        const uint32_t key = range_key(g[k]);
+        acc.min_key = key < acc.min_key ? key : acc.min_key;
+        if (WITH_GS) {
             const int t = code_q(code_of(w, k), cd) - 1;
             const float gt = g[k] * (float)t;
-            grad_s = grad_s + gt;
+            acc.grad_s = acc.grad_s + gt;
         }
     }
 }
@@ -66,160 +107,297 @@ __device__ __forceinline__ float tree_sum(float a) {
     // lg[lid] += lg[lid + s] for s = 32..1 (kernels/compact_counter.cl:88-91)
 #pragma unroll
     for (int s = kWave / 2; s > 0; s >>= 1) a = a + __shfl_down(a, s, kWave);
+    return __shfl(a, 0, kWave);
+}
+
+__device__ __forceinline__ uint32_t wave_min(uint32_t a) {
+#pragma unroll
+    for (int s = kWave / 2; s > 0; s >>= 1) {
+        const uint32_t b = (uint32_t)__shfl_xor((int)a, s, kWave);
+        a = b < a ? b : a;
+    }
     return a;
 }
 
-__device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], const RowConsts& rc,
-                                               const UpdateArgs& a, uint32_t elem0) {
+struct RowCtx {
+    TickConsts tc;
+    bool fast_div;  // wave-uniform
+};
+
+// Tree reduction, row epilogue, commit of v/scale, and the per-row c_reb table.
+template <bool WITH_GS>
+__device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTensor& t, int row, int lane,
+                                             const RowAcc& acc, Luts& l) {
+    const float g_sq = tree_sum(acc.g_sq);
+    const float grad_s = WITH_GS ? tree_sum(acc.grad_s) : 0.0f;
+    const uint32_t min_key = wave_min(acc.min_key);
+    const float s_old = t.scale[row];
+    const float v_old = t.v[row];
+    const RowStats rs = finish_row_stats(g_sq, grad_s, v_old, s_old, t.in_features, a.lr_scale,
+                                         a.rms_beta, a.rms_eps);
+    if (lane == 0) {
+        t.v[row] = rs.v_new;
+        t.scale[row] = rs.scale_new;  // commit (kernels/basic.cl:6-9); s_old stays in a register
+    }
+    __syncthreads();  // the previous row's ticks have finished reading c_reb
+    l.c_reb[lane] = c_reb_entry((uint32_t)lane, a.cd, s_old / rs.scale_new);
+    __syncthreads();
+    RowCtx rc;
+    rc.tc.dn = rs.denom;
+    rc.tc.r = 1.0f / rs.denom;
+    rc.tc.k = a.cd.Cf / rs.scale_new;
+    rc.tc.neg_lr = -t.lr;
+    rc.tc.neg_lim_neg = -(float)a.geom.lim_neg;
+    rc.tc.lim_pos = (float)a.geom.lim_pos;
+    rc.tc.seed = t.seed;
+    rc.tc.shift = a.geom.shift;
+    rc.fast_div = __builtin_amdgcn_readfirstlane(row_takes_fast_division(rs.denom, g_sq, min_key) ? 1 : 0) != 0;
+    return rc;
+}
+
+template <bool FAST_DIV>
+__device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], const TickConsts& tc,
+                                               const Luts& l, uint32_t elem0) {
     uint32_t nw = 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const uint32_t nc = tick_code(code_of(w, k), g[k], rc, a.seed, elem0 + (uint32_t)k, a.cd);
-        nw |= (nc & 0x3fu) << (6 * k);
+        const uint32_t nc = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, elem0 + (uint32_t)k, l.c_reb, l.q_off, l.fin);
+        nw |= nc << (6 * k);
     }
     return nw;
 }
 
-__device__ __forceinline__ RowConsts finish_row(const UpdateArgs& a, int row, int lane, float g_sq,
-                                                float grad_s, bool with_gs) {
-    g_sq = tree_sum(g_sq);
-    g_sq = __shfl(g_sq, 0, kWave);
-    if (with_gs) {
-        grad_s = tree_sum(grad_s);
-        grad_s = __shfl(grad_s, 0, kWave);
-    } else {
-        grad_s = 0.0f;
+// Tick pass over a row re-read from memory with byte-granular state access: the fallback for
+// rows of any length and alignment, and for rows that need the plain division.
+__device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, int lane, const TickConsts& tc,
+                                               const Luts& l) {
+    const int gpr = t.in_features >> 2;
+    const float* g_row = t.grad_w + (size_t)row * t.in_features;
+    uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
+    for (int gi = lane; gi < gpr; gi += kWave) {
+        float g[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) g[k] = g_row[4 * gi + k];
+        const uint32_t nw = tick_group<false>(load_group(s_row + 3 * gi), g, tc, l, row_elem + 4u * (uint32_t)gi);
+        store_group(s_row + 3 * gi, nw);
     }
-    const float s_old = a.scale[row];
-    const float v_old = a.v[row];
-    const RowStats rs = finish_row_stats(g_sq, grad_s, v_old, s_old, a.in_features, a.lr_scale,
-                                         a.rms_beta, a.rms_eps);
-    if (lane == 0) {
-        a.v[row] = rs.v_new;
-        a.scale[row] = rs.scale_new;  // commit (kernels/basic.cl:6-9); s_old stays in a register
-    }
-    RowConsts rc;
-    rc.dn = rs.denom;
-    rc.k = a.cd.Cf / rs.scale_new;
-    rc.ratio = s_old / rs.scale_new;
-    rc.neg_lr = -a.lr;
-    return rc;
 }
 
-// Register-resident rows: gpr <= 64 * ITERS.  grad_w must be 16-byte aligned.
+// One row, held in registers: gpr <= 64 * ITERS, grad_w 16-byte aligned, and the row is not
+// the last of its tensor (so reading one byte past any of its groups stays inside the state).
+// All loads of the row are issued back to back with no branch between them: lanes past the end
+// of the row re-read its last group and are masked out of the sums and of the apply.
 template <int ITERS, bool WITH_GS>
-__global__ __launch_bounds__(kWave* kWavesPerBlock) void update_rows_kernel(UpdateArgs a) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int row = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-    if (row >= a.out_features) return;
-    const float4* g_row = reinterpret_cast<const float4*>(a.grad_w + (size_t)row * a.in_features);
-    uint8_t* s_row = a.state + (size_t)row * a.gpr * 3;
+__device__ __forceinline__ void update_row_resident(const BatchArgs& a, const UpdateTensor& t, int row,
+                                                    int lane, Luts& luts) {
+    constexpr bool kKeepWords = ITERS <= 24;  // longer rows re-read their state words (L2 hits)
+    const int gpr = t.in_features >> 2;
+    const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
+    uint8_t* s_row = t.state + (size_t)row * gpr * 3;
 
-    float g[ITERS][4];
-    uint32_t w[ITERS];
+    float4 q[ITERS];
+    uint32_t w[kKeepWords ? ITERS : 1];
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const int gi = lane + kWave * j;
-        if (gi < a.gpr) {
-            const float4 q = g_row[gi];
-            g[j][0] = q.x; g[j][1] = q.y; g[j][2] = q.z; g[j][3] = q.w;
-            w[j] = load_group(s_row + 3 * gi);
-        } else {
-            g[j][0] = g[j][1] = g[j][2] = g[j][3] = 0.0f;
-            w[j] = 0u;
+        const int gc = gi < gpr ? gi : gpr - 1;
+        q[j] = g_row[gc];
+        if (kKeepWords || WITH_GS) {
+            const uint32_t word = load_group_dword(s_row + 3 * gc);
+            if (kKeepWords) w[j] = word;
         }
     }
-    float g_sq = 0.0f, grad_s = 0.0f;
+    RowAcc acc;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
-        // a padded group adds +0.0 (squares) and -0.0 (0 * t, t = -1): both leave the sums unchanged
-        accumulate(g_sq, grad_s, g[j], w[j], a.cd, WITH_GS);
+        const bool live = lane + kWave * j < gpr;
+        // a masked group adds +0.0 (squares) and -+0.0 (0 * t): both leave the sums unchanged
+        const float g[4] = {live ? q[j].x : 0.0f, live ? q[j].y : 0.0f, live ? q[j].z : 0.0f,
+                            live ? q[j].w : 0.0f};
+        uint32_t word = 0;
+        if (WITH_GS) {
+            const int gi = lane + kWave * j;
+            word = kKeepWords ? w[j] : load_group_dword(s_row + 3 * (gi < gpr ? gi : gpr - 1));
+        }
+        accumulate<WITH_GS>(acc, g, word, a.cd);
     }
-    const RowConsts rc = finish_row(a, row, lane, g_sq, grad_s, WITH_GS);
-    const uint32_t row_elem = (uint32_t)row * (uint32_t)a.in_features;
+    const RowCtx rc = finish_row<WITH_GS>(a, t, row, lane, acc, luts);
+    if (!rc.fast_div) {
+        apply_streamed(t, row, lane, rc.tc, luts);
+        return;
+    }
+    const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const int gi = lane + kWave * j;
-        if (gi < a.gpr) {
-            const uint32_t nw = tick_group(w[j], g[j], rc, a, row_elem + 4u * (uint32_t)gi);
+        if (gi < gpr) {
+            const float g[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
+            const uint32_t word = kKeepWords ? w[j] : load_group_dword(s_row + 3 * gi);
+            const uint32_t nw = tick_group<true>(word, g, rc.tc, luts, row_elem + 4u * (uint32_t)gi);
             store_group(s_row + 3 * gi, nw);
         }
     }
 }
 
-// Any row length, any alignment: the row is read twice (the second read hits L2).
+// One row of any length and alignment: read twice (the second read hits L2).
 template <bool WITH_GS>
-__global__ __launch_bounds__(kWave* kWavesPerBlock) void update_rows_generic_kernel(UpdateArgs a) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int row = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-    if (row >= a.out_features) return;
-    const float* g_row = a.grad_w + (size_t)row * a.in_features;
-    uint8_t* s_row = a.state + (size_t)row * a.gpr * 3;
-
-    float g_sq = 0.0f, grad_s = 0.0f;
-    for (int gi = lane; gi < a.gpr; gi += kWave) {
+__device__ __forceinline__ void update_row_streamed(const BatchArgs& a, const UpdateTensor& t, int row,
+                                                    int lane, Luts& luts) {
+    const int gpr = t.in_features >> 2;
+    const float* g_row = t.grad_w + (size_t)row * t.in_features;
+    const uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    RowAcc acc;
+    for (int gi = lane; gi < gpr; gi += kWave) {
         float g[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) g[k] = g_row[4 * gi + k];
-        accumulate(g_sq, grad_s, g, load_group(s_row + 3 * gi), a.cd, WITH_GS);
+        accumulate<WITH_GS>(acc, g, load_group(s_row + 3 * gi), a.cd);
     }
-    const RowConsts rc = finish_row(a, row, lane, g_sq, grad_s, WITH_GS);
-    const uint32_t row_elem = (uint32_t)row * (uint32_t)a.in_features;
-    for (int gi = lane; gi < a.gpr; gi += kWave) {
-        float g[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) g[k] = g_row[4 * gi + k];
-        const uint32_t nw = tick_group(load_group(s_row + 3 * gi), g, rc, a, row_elem + 4u * (uint32_t)gi);
-        store_group(s_row + 3 * gi, nw);
+    const RowCtx rc = finish_row<WITH_GS>(a, t, row, lane, acc, luts);
+    apply_streamed(t, row, lane, rc.tc, luts);
+}
+
+// Minimum waves per SIMD the compiler must leave room for: the tick arithmetic has long
+// dependent chains, so the row's registers are budgeted to keep 3-4 waves resident for short
+// rows and 2 for the longest.
+constexpr int min_waves(int iters) { return iters <= 8 ? 4 : (iters <= 16 ? 3 : 2); }
+
+template <int ITERS, bool WITH_GS>
+__global__ __launch_bounds__(kThreads, min_waves(ITERS)) void update_rows_kernel(BatchArgs a) {
+    __shared__ Luts luts;
+    build_luts(luts, a.cd, a.geom);
+    const int lane = threadIdx.x;
+    // everything that selects the row depends on blockIdx only, so it lives in scalar registers
+    const int wave = blockIdx.x;
+    const int stride = gridDim.x;
+    int ti = 0;
+    for (int grow_v = wave; grow_v < a.total_rows; grow_v += stride) {
+        // readfirstlane pins the row and tensor index into scalar registers, so the descriptor
+        // fields below are scalar loads from the kernel-argument segment
+        const int grow = __builtin_amdgcn_readfirstlane(grow_v);
+        ti = __builtin_amdgcn_readfirstlane(ti);
+        while (grow >= a.t[ti].row_start + a.t[ti].out_features) ++ti;  // monotonic
+        ti = __builtin_amdgcn_readfirstlane(ti);
+        const UpdateTensor t = a.t[ti];
+        const int row = grow - t.row_start;
+        // the tensor's last row goes through the byte-granular path: its last group has no
+        // byte after it for the 4-byte state load
+        if (ITERS > 0 && row != t.out_features - 1)
+            update_row_resident<(ITERS > 0 ? ITERS : 1), WITH_GS>(a, t, row, lane, luts);
+        else
+            update_row_streamed<WITH_GS>(a, t, row, lane, luts);
     }
 }
 
+int device_cu_count() {
+    static int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+        return n;
+    }();
+    return cus;
+}
+
+template <int ITERS, bool WITH_GS>
+hipError_t launch_variant(hipStream_t stream, const BatchArgs& a) {
+    static int blocks_per_cu = [] {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_kernel<ITERS, WITH_GS>, kThreads, 0) != hipSuccess ||
+            n <= 0)
+            n = 2;
+        return n;
+    }();
+    const int want = (a.total_rows + kWavesPerBlock - 1) / kWavesPerBlock;
+    const int resident = device_cu_count() * blocks_per_cu;
+    const dim3 grid(want < resident ? want : resident);
+    hipLaunchKernelGGL((update_rows_kernel<ITERS, WITH_GS>), grid, dim3(kThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
 template <int ITERS>
-void launch_rows(const UpdateArgs& a, hipStream_t stream) {
-    const dim3 grid((a.out_features + kWavesPerBlock - 1) / kWavesPerBlock);
-    const dim3 block(kWave * kWavesPerBlock);
-    if (a.lr_scale != 0.0f)
-        hipLaunchKernelGGL((update_rows_kernel<ITERS, true>), grid, block, 0, stream, a);
-    else
-        hipLaunchKernelGGL((update_rows_kernel<ITERS, false>), grid, block, 0, stream, a);
+hipError_t launch_iters(hipStream_t stream, const BatchArgs& a) {
+    return a.lr_scale != 0.0f ? launch_variant<ITERS, true>(stream, a) : launch_variant<ITERS, false>(stream, a);
+}
+
+// Register-resident variant that fits a row of `in_features` (0 = streamed fallback).
+int iters_class(const UpdateTensor& t) {
+    const int iters = ((t.in_features >> 2) + kWave - 1) / kWave;
+    const bool aligned = (reinterpret_cast<uintptr_t>(t.grad_w) & 15u) == 0;
+    if (!aligned) return 0;
+    static const int classes[] = {1, 2, 3, 4, 8, 12, 16, 24, 32, 43};
+    for (int c : classes)
+        if (iters <= c) return c;
+    return 0;
+}
+
+hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
+    switch (cls) {
+        case 1: return launch_iters<1>(stream, a);
+        case 2: return launch_iters<2>(stream, a);
+        case 3: return launch_iters<3>(stream, a);
+        case 4: return launch_iters<4>(stream, a);
+        case 8: return launch_iters<8>(stream, a);
+        case 12: return launch_iters<12>(stream, a);
+        case 16: return launch_iters<16>(stream, a);
+        case 24: return launch_iters<24>(stream, a);
+        case 32: return launch_iters<32>(stream, a);
+        case 43: return launch_iters<43>(stream, a);
+        default: return launch_iters<0>(stream, a);
+    }
 }
 
 }  // namespace
 
-// Enqueues the update-only step.  Arguments are already validated by the caller.
+// Enqueues the update-only step for `n` tensors (already validated).  Tensors are grouped by
+// the register-resident variant their row length needs; each group goes out in launches of at
+// most kMaxUpdateBatch tensors.
+hipError_t launch_update_batch(hipStream_t stream, const UpdateTensor* tensors, size_t n, int C,
+                               float lr_scale, float rms_beta, float rms_eps) {
+    BatchArgs a;
+    a.cd = make_codec(C);
+    a.geom = lut_geom(a.cd);
+    a.lr_scale = lr_scale; a.rms_beta = rms_beta; a.rms_eps = rms_eps;
+    std::vector<int> cls(n);
+    std::vector<char> done(n, 0);
+    for (size_t i = 0; i < n; ++i) cls[i] = iters_class(tensors[i]);
+    for (size_t i = 0; i < n; ++i) {
+        if (done[i]) continue;
+        a.n_tensors = 0;
+        a.total_rows = 0;
+        for (size_t j = i; j < n; ++j) {
+            if (done[j] || cls[j] != cls[i]) continue;
+            // total_rows stays below 2^31: flush before the row space of one launch gets there
+            if (a.n_tensors == kMaxUpdateBatch || a.total_rows > (1 << 30) - tensors[j].out_features) {
+                const hipError_t e = launch_class(stream, cls[i], a);
+                if (e != hipSuccess) return e;
+                a.n_tensors = 0;
+                a.total_rows = 0;
+            }
+            a.t[a.n_tensors] = tensors[j];
+            a.t[a.n_tensors].row_start = a.total_rows;
+            a.total_rows += tensors[j].out_features;
+            ++a.n_tensors;
+            done[j] = 1;
+        }
+        if (a.n_tensors > 0) {
+            const hipError_t e = launch_class(stream, cls[i], a);
+            if (e != hipSuccess) return e;
+        }
+    }
+    return hipSuccess;
+}
+
 hipError_t launch_update_dense(hipStream_t stream, uint8_t* state, float* scale, float* v,
                                const float* grad_w, int C, int in_features, int out_features,
                                float lr, float lr_scale, float rms_beta, float rms_eps,
                                uint32_t seed) {
-    UpdateArgs a;
-    a.state = state; a.scale = scale; a.v = v; a.grad_w = grad_w;
-    a.cd = make_codec(C);
-    a.in_features = in_features; a.out_features = out_features;
-    a.gpr = in_features / 4;
-    a.lr = lr; a.lr_scale = lr_scale; a.rms_beta = rms_beta; a.rms_eps = rms_eps;
-    a.seed = seed;
-
-    const int iters = (a.gpr + kWave - 1) / kWave;
-    const bool aligned = (reinterpret_cast<uintptr_t>(grad_w) & 15u) == 0;
-    if (aligned && iters <= 1) launch_rows<1>(a, stream);
-    else if (aligned && iters <= 2) launch_rows<2>(a, stream);
-    else if (aligned && iters <= 3) launch_rows<3>(a, stream);
-    else if (aligned && iters <= 4) launch_rows<4>(a, stream);
-    else if (aligned && iters <= 8) launch_rows<8>(a, stream);
-    else if (aligned && iters <= 12) launch_rows<12>(a, stream);
-    else if (aligned && iters <= 16) launch_rows<16>(a, stream);
-    else if (aligned && iters <= 24) launch_rows<24>(a, stream);
-    else if (aligned && iters <= 32) launch_rows<32>(a, stream);
-    else if (aligned && iters <= 43) launch_rows<43>(a, stream);
-    else {
-        const dim3 grid((a.out_features + kWavesPerBlock - 1) / kWavesPerBlock);
-        const dim3 block(kWave * kWavesPerBlock);
-        if (a.lr_scale != 0.0f)
-            hipLaunchKernelGGL((update_rows_generic_kernel<true>), grid, block, 0, stream, a);
-        else
-            hipLaunchKernelGGL((update_rows_generic_kernel<false>), grid, block, 0, stream, a);
-    }
-    return hipGetLastError();
+    UpdateTensor t;
+    t.state = state; t.scale = scale; t.v = v; t.grad_w = grad_w;
+    t.in_features = in_features; t.out_features = out_features;
+    t.row_start = 0; t.seed = seed; t.lr = lr; t.pad = 0;
+    return launch_update_batch(stream, &t, 1, C, lr_scale, rms_beta, rms_eps);
 }
 
 }  // namespace mcc

@@ -8,6 +8,23 @@
 
 namespace mcc {
 
+// One counter tensor of an update-only batch (device pointers).
+struct UpdateTensor {
+    uint8_t* state;
+    float* scale;
+    float* v;
+    const float* grad_w;
+    int in_features, out_features;
+    int row_start;  // first row of this tensor in the launch's concatenated row space
+    uint32_t seed;
+    float lr;
+    int pad;
+};
+constexpr int kMaxUpdateBatch = 64;  // tensors per launch: the descriptors travel as kernel arguments
+
+hipError_t launch_update_batch(hipStream_t stream, const UpdateTensor* tensors, size_t n, int C,
+                               float lr_scale, float rms_beta, float rms_eps);
+
 hipError_t launch_update_dense(hipStream_t stream, uint8_t* state, float* scale, float* v,
                                const float* grad_w, int C, int in_features, int out_features,
                                float lr, float lr_scale, float rms_beta, float rms_eps,

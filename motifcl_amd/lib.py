@@ -13,6 +13,8 @@ SIGNATURES = {
     "mcc_device_name": (ctypes.c_char_p, []),
     "mcc_compact_counter_apply_update_dense": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
+    "mcc_compact_counter_apply_update_dense_batched": (
+        ctypes.c_int, [_vp, _vp, _sz, _sz, _f, _f, _f]),
     "mcc_compact_counter_fused_workspace_nbytes": (_sz, [_sz, _sz, _sz]),
     "mcc_compact_counter_apply_update_fused": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
@@ -38,6 +40,15 @@ SIGNATURES = {
     "mcc_profiler_query": (ctypes.c_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_uint64)]),
 }
+
+
+
+class CounterTensor(ctypes.Structure):
+    """struct mcc_counter_tensor of include/motifcl_amd.h."""
+    _fields_ = [("state", _vp), ("state_nbytes", _sz), ("scale", _vp), ("scale_nbytes", _sz),
+                ("v", _vp), ("v_nbytes", _sz), ("grad_w", _vp), ("grad_w_nbytes", _sz),
+                ("in_features", _sz), ("out_features", _sz), ("lr", _f), ("seed", _u32)]
+
 
 _lib = None
 

@@ -32,6 +32,38 @@ def apply_update_dense(state, scale, v, grad_w, C, lr, lr_scale, rms_beta, rms_e
         lr, lr_scale, rms_beta, rms_eps, seed & 0xFFFFFFFF))
 
 
+class UpdateBatch:
+    """A reusable descriptor list for apply_update_dense_batched: tensors are
+    (state, scale, v, grad_w) device tensors with grad_w of shape [out, in]."""
+
+    def __init__(self, tensors, lr, seeds):
+        self._keep = list(tensors)
+        n = len(self._keep)
+        self.array = (_lib.CounterTensor * n)()
+        for i, (state, scale, v, grad_w) in enumerate(self._keep):
+            out_features, in_features = grad_w.shape
+            d = self.array[i]
+            d.state, d.state_nbytes = _buf(state, torch.uint8)
+            d.scale, d.scale_nbytes = _buf(scale, torch.float32)
+            d.v, d.v_nbytes = _buf(v, torch.float32)
+            d.grad_w, d.grad_w_nbytes = _buf(grad_w, torch.float32)
+            d.in_features, d.out_features = in_features, out_features
+            d.lr = lr[i] if isinstance(lr, (list, tuple)) else lr
+            d.seed = seeds[i] & 0xFFFFFFFF
+        self.n = n
+
+    def set_seeds(self, seeds):
+        for i in range(self.n):
+            self.array[i].seed = seeds[i] & 0xFFFFFFFF
+
+
+def apply_update_dense_batched(batch, C, lr_scale, rms_beta, rms_eps):
+    """In-place update-only step of every tensor of an UpdateBatch, one call."""
+    L = _lib.load()
+    _lib.check(L.mcc_compact_counter_apply_update_dense_batched(
+        _stream(), batch.array, batch.n, C, lr_scale, rms_beta, rms_eps))
+
+
 def fused_workspace_nbytes(in_features, out_features, batch):
     return int(_lib.load().mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch))
 

@@ -1,0 +1,100 @@
+// CPU build of the kernels' tick arithmetic (motifcl_amd/csrc/counter_math.hpp) checked
+// against the oracle's literal restatement (oracle/counter_oracle.c) on millions of
+// inputs, including every code, every C, integral / near-integral / huge / tiny values.
+// Build: g++ -O2 -ffp-contract=off -fopenmp check_tick_math.cpp ../../oracle/counter_oracle.c-as-lib
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../../motifcl_amd/csrc/counter_math.hpp"
+
+extern "C" int oracle_tick_code(int code, float gw, float s_old, float s_new, float dn, int C,
+                                float lr, uint32_t seed, uint32_t elem);
+
+static uint64_t rng_state = 0x9E3779B97F4A7C15ull;
+static uint64_t next_u64() {
+    rng_state ^= rng_state << 13; rng_state ^= rng_state >> 7; rng_state ^= rng_state << 17;
+    return rng_state;
+}
+static double uni() { return (next_u64() >> 11) * (1.0 / 9007199254740992.0); }
+static float log_uniform(double lo, double hi) { return (float)std::exp(std::log(lo) + uni() * (std::log(hi) - std::log(lo))); }
+
+int main(int argc, char** argv) {
+    const long per_c = argc > 1 ? std::atol(argv[1]) : 2000000;
+    long mismatches = 0, checked = 0, n_fast = 0;
+    for (int C = 1; C <= 11; ++C) {
+        const mcc::Codec cd = mcc::make_codec(C);
+        const mcc::LutGeom g = mcc::lut_geom(cd);
+        if ((g.width << g.shift) > mcc::kLutFinMaxBytes) { std::printf("LUT too large for C=%d\n", C); return 2; }
+        std::vector<uint8_t> fin(g.width << g.shift);
+        std::vector<int> q_off(64);
+        std::vector<float> c_reb(64);
+        for (uint32_t code = 0; code < 64; ++code) q_off[code] = mcc::q_off_entry(code, cd, g);
+        for (int i = 0; i < (g.width << g.shift); ++i) mcc::fill_fin_entry(i, cd, g, fin.data());
+        // (code * magic) >> 16 == code / lv
+        for (uint32_t code = 0; code < 64; ++code)
+            if (mcc::code_q(code, cd) != (int)code / cd.lv) { std::printf("magic division fails C=%d code=%u\n", C, code); return 2; }
+        auto make_tc = [&](float dn, float s_old, float s_new, float lr, uint32_t seed) {
+            mcc::TickConsts tc;
+            tc.dn = dn; tc.r = 1.0f / dn; tc.k = cd.Cf / s_new; tc.neg_lr = -lr;
+            tc.neg_lim_neg = -(float)g.lim_neg; tc.lim_pos = (float)g.lim_pos;
+            tc.seed = seed; tc.shift = g.shift;
+            for (uint32_t code = 0; code < 64; ++code) c_reb[code] = mcc::c_reb_entry(code, cd, s_old / s_new);
+            return tc;
+        };
+        const float lrs[] = {3e-3f, 0.05f, 1.0f, 16.0f, 100.0f, 0.0f};
+        for (long it = 0; it < per_c; ++it) {
+            const int code = (int)(next_u64() % 64);
+            const int mode = (int)(next_u64() % 8);
+            float lr = lrs[next_u64() % 6];
+            float dn = (next_u64() & 15) ? log_uniform(1e-8, 1e3) : log_uniform(1e-30, 1e30), s_old = log_uniform(1e-5, 10.0), s_new = log_uniform(1e-5, 10.0);
+            float gw;
+            if (mode == 0) { s_new = s_old; }                       // lr_scale = 0: ratio is exactly 1
+            if (mode == 1) gw = 0.0f;
+            else if (mode == 2) gw = (uni() < 0.5 ? -1.f : 1.f) * log_uniform(1e-44, 1e-6);
+            else if (mode == 3) gw = (uni() < 0.5 ? -1.f : 1.f) * log_uniform(1e3, 1e12);
+            else gw = (float)((uni() - 0.5) * 2.0) * log_uniform(1e-6, 10.0);
+            if (mode == 4 || mode == 5) {
+                // integral or near-integral val: tick = -gw exactly (dn = 64, lr = 16, C/s_new = 4)
+                dn = 64.0f; lr = 16.0f; s_new = (float)C / 4.0f; s_old = s_new;
+                gw = (float)((long)(next_u64() % 401) - 200);
+                if (mode == 5) gw = std::nextafterf(gw, uni() < 0.5 ? -1e9f : 1e9f);
+            }
+            // the reference's conversions are undefined from |val| = 2^31 on: stay inside the contract
+            const float bound = std::fabs((lr * (gw / dn)) * ((float)C / s_new)) + 64.0f * (s_old / s_new);
+            if (!(bound < 2.0e9f)) continue;
+            const uint32_t seed = (uint32_t)next_u64(), elem = (uint32_t)next_u64();
+            const mcc::TickConsts tc = make_tc(dn, s_old, s_new, lr, seed);
+            // the kernel decides per row from the row's sum of squares and smallest non-zero
+            // magnitude; a one-element "row" exercises both branches of that decision
+            const bool fast = mcc::row_takes_fast_division(dn, (next_u64() & 7) ? gw * gw * 64.0f : 0x1p110f,
+                                                           mcc::range_key(gw));
+            n_fast += fast;
+            const uint32_t got = fast
+                ? mcc::tick_code<true>((uint32_t)code, gw, tc, elem, c_reb.data(), q_off.data(), fin.data())
+                : mcc::tick_code<false>((uint32_t)code, gw, tc, elem, c_reb.data(), q_off.data(), fin.data());
+            const int exp = oracle_tick_code(code, gw, s_old, s_new, dn, C, lr, seed, elem);
+            ++checked;
+            if ((int)got != exp) {
+                if (mismatches < 10)
+                    std::printf("MISMATCH C=%d code=%d gw=%a dn=%a s_old=%a s_new=%a lr=%a seed=%u elem=%u got=%u exp=%d\n",
+                                C, code, gw, dn, s_old, s_new, lr, seed, elem, got, exp);
+                ++mismatches;
+            }
+        }
+        // every (q, total) pair of the table against the oracle through exact integer ticks
+        for (int code = 0; code < 64; ++code)
+            for (int gi = -4 * 64; gi <= 4 * 64; ++gi) {
+                const float s = (float)C / 4.0f;
+                const mcc::TickConsts tc = make_tc(64.0f, s, s, 16.0f, 1u);
+                const uint32_t got = mcc::tick_code<true>((uint32_t)code, (float)gi, tc, 2u, c_reb.data(), q_off.data(), fin.data());
+                const int exp = oracle_tick_code(code, (float)gi, s, s, 64.0f, C, 16.0f, 1u, 2u);
+                ++checked;
+                if ((int)got != exp) { if (mismatches < 10) std::printf("TABLE MISMATCH C=%d code=%d g=%d got=%u exp=%d\n", C, code, gi, got, exp); ++mismatches; }
+            }
+    }
+    std::printf("checked %ld ticks (%ld through the reciprocal division), %ld mismatches\n", checked, n_fast, mismatches);
+    return mismatches == 0 ? 0 : 1;
+}

@@ -113,6 +113,51 @@ def test_update_dense_misaligned_gradient_pointer(ops, oracle):
     assert_bit_exact([host(t) for t in d], oracle.update_dense(state, scale, v, G, C, 3e-3, 0.01, 0.9, 1e-3, 42))
 
 
+def test_update_dense_batched_matches_per_tensor_oracle(ops, oracle):
+    # mixed row lengths (several kernel variants, the streamed fallback, a misaligned gradient)
+    # and more tensors than one launch carries (64): every tensor must equal its own
+    # single-tensor oracle result
+    shapes = [(40, 288), (17, 4096), (9, 260), (6, 11008), (33, 768), (5, 16384), (12, 2048)]
+    shapes += [(3 + (i % 5), 64 * (1 + i % 3)) for i in range(70)]
+    C, hp = 11, dict(lr_scale=0.01, rms_beta=0.9, rms_eps=1e-3)
+    cases, dev_tensors, lrs, seeds = [], [], [], []
+    for i, (n_out, n_in) in enumerate(shapes):
+        _, state, G, scale, v = synth.counter_case(1000 + i, n_out, n_in, C, oracle=oracle)
+        if i == 2:  # 4-byte aligned gradient view
+            buf = torch.empty(n_out * n_in + 1, dtype=torch.float32, device="cuda")
+            g_dev = buf[1:].view(n_out, n_in)
+            g_dev.copy_(dev(G))
+        else:
+            g_dev = dev(G)
+        cases.append((state, scale, v, G))
+        dev_tensors.append((dev(state), dev(scale), dev(v), g_dev))
+        lrs.append(3e-3 * (1 + i % 3))
+        seeds.append(777 + 13 * i)
+    batch = ops.UpdateBatch(dev_tensors, lrs, seeds)
+    ops.apply_update_dense_batched(batch, C, hp["lr_scale"], hp["rms_beta"], hp["rms_eps"])
+    torch.cuda.synchronize()
+    for i, (state, scale, v, G) in enumerate(cases):
+        exp = oracle.update_dense(state, scale, v, G, C, lrs[i], hp["lr_scale"], hp["rms_beta"],
+                                  hp["rms_eps"], seeds[i])
+        assert_bit_exact([host(t) for t in dev_tensors[i][:3]], exp)
+
+
+def test_tiny_and_huge_gradients_take_the_exact_division(ops, oracle):
+    # rows whose gradients leave the range of the reciprocal-based division (denormal and
+    # 1e-30 entries next to ordinary ones; a row with a 1e25 entry) must still be bit-exact
+    n_out, n_in, C = 8, 512, 11
+    _, state, G, scale, v = synth.counter_case(31, n_out, n_in, C, oracle=oracle)
+    G[0, ::3] = 1e-42
+    G[1, ::5] = -3e-31
+    G[2, 7] = 1e25
+    G[3] *= 1e-20
+    G[4] = 0.0
+    G[5, ::2] = 0.0
+    d = [dev(state), dev(scale), dev(v)]
+    ops.apply_update_dense(*d, dev(G), C, 0.5, 0.0, 0.9, 0.0, 99)
+    assert_bit_exact([host(t) for t in d], oracle.update_dense(state, scale, v, G, C, 0.5, 0.0, 0.9, 0.0, 99))
+
+
 def test_integer_ticks_closed_form_on_gpu(ops, oracle):
     # tick = -g exactly (see tests/test_oracle_pins.py): z = C*t + c moves by -g or saturates
     C = 11
