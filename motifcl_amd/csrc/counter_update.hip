@@ -48,9 +48,9 @@ struct BatchArgs {
 // Per-workgroup tables in LDS (see counter_math.hpp).  fin and q_off depend on C only and are
 // built once per launch; c_reb depends on the row's scale ratio and is rebuilt per row.
 struct Luts {
-    uint8_t fin[kLutFinMaxBytes];
-    int q_off[64];
+    int q_off[64];   // first, so that the decode reads need no base-address add
     float c_reb[64];
+    uint8_t fin[kLutFinMaxBytes];
 };
 
 __device__ __forceinline__ void build_luts(Luts& l, const Codec& cd, const LutGeom& geom) {
@@ -103,20 +103,37 @@ __device__ __forceinline__ void accumulate(RowAcc& acc, const float g[4], uint32
     }
 }
 
-__device__ __forceinline__ float tree_sum(float a) {
-    // lg[lid] += lg[lid + s] for s = 32..1 (kernels/compact_counter.cl:88-91)
-#pragma unroll
-    for (int s = kWave / 2; s > 0; s >>= 1) a = a + __shfl_down(a, s, kWave);
-    return __shfl(a, 0, kWave);
+// lane l <- value of lane l + N of the same 16-lane row (DPP row_shl); lanes whose source
+// falls outside the row keep their own value, which no later step of the tree reads.
+template <int N>
+__device__ __forceinline__ uint32_t row_from_above(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x100 + N, 0xf, 0xf, false);
 }
 
-__device__ __forceinline__ uint32_t wave_min(uint32_t a) {
-#pragma unroll
-    for (int s = kWave / 2; s > 0; s >>= 1) {
-        const uint32_t b = (uint32_t)__shfl_xor((int)a, s, kWave);
-        a = b < a ? b : a;
-    }
-    return a;
+// lg[lid] += lg[lid + s] for s = 32, 16, 8, 4, 2, 1 (kernels/compact_counter.cl:88-91): the
+// same pairing and order as the reference's LDS tree.  The two steps that cross 16-lane rows
+// go through the LDS crossbar, the other four are DPP operands of the add itself.
+__device__ __forceinline__ float tree_sum(float a, int lane) {
+    a = a + __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute((lane + 32) << 2, (int)__float_as_uint(a)));
+    a = a + __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute((lane + 16) << 2, (int)__float_as_uint(a)));
+    a = a + __uint_as_float(row_from_above<8>(__float_as_uint(a)));
+    a = a + __uint_as_float(row_from_above<4>(__float_as_uint(a)));
+    a = a + __uint_as_float(row_from_above<2>(__float_as_uint(a)));
+    a = a + __uint_as_float(row_from_above<1>(__float_as_uint(a)));
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(a)));
+}
+
+__device__ __forceinline__ uint32_t umin(uint32_t a, uint32_t b) { return b < a ? b : a; }
+
+// Minimum over the wave, taken at lane 0 (same pairing as tree_sum; any order would do).
+__device__ __forceinline__ uint32_t wave_min(uint32_t a, int lane) {
+    a = umin(a, (uint32_t)__builtin_amdgcn_ds_bpermute((lane + 32) << 2, (int)a));
+    a = umin(a, (uint32_t)__builtin_amdgcn_ds_bpermute((lane + 16) << 2, (int)a));
+    a = umin(a, row_from_above<8>(a));
+    a = umin(a, row_from_above<4>(a));
+    a = umin(a, row_from_above<2>(a));
+    a = umin(a, row_from_above<1>(a));
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)a);
 }
 
 struct RowCtx {
@@ -128,9 +145,9 @@ struct RowCtx {
 template <bool WITH_GS>
 __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTensor& t, int row, int lane,
                                              const RowAcc& acc, Luts& l) {
-    const float g_sq = tree_sum(acc.g_sq);
-    const float grad_s = WITH_GS ? tree_sum(acc.grad_s) : 0.0f;
-    const uint32_t min_key = wave_min(acc.min_key);
+    const float g_sq = tree_sum(acc.g_sq, lane);
+    const float grad_s = WITH_GS ? tree_sum(acc.grad_s, lane) : 0.0f;
+    const uint32_t min_key = wave_min(acc.min_key, lane);
     const float s_old = t.scale[row];
     const float v_old = t.v[row];
     const RowStats rs = finish_row_stats(g_sq, grad_s, v_old, s_old, t.in_features, a.lr_scale,
@@ -184,41 +201,43 @@ __device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, i
     }
 }
 
-// One row, held in registers: gpr <= 64 * ITERS, grad_w 16-byte aligned, and the row is not
-// the last of its tensor (so reading one byte past any of its groups stays inside the state).
-// All loads of the row are issued back to back with no branch between them: lanes past the end
-// of the row re-read its last group and are masked out of the sums and of the apply.
+// One row, held in registers: ITERS == ceil(gpr / 64) exactly, grad_w 16-byte aligned, and the
+// row is not the last of its tensor (so reading one byte past any of its groups stays inside
+// the state).  Every iteration but the last covers 64 full groups, so its loads, sums and
+// stores need no masks and all addresses are one per-lane base plus a compile-time offset;
+// in the last iteration lanes past the end of the row re-read the row's last group and are
+// masked out of the sums and of the store.  All loads are issued back to back.
 template <int ITERS, bool WITH_GS>
 __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const UpdateTensor& t, int row,
                                                     int lane, Luts& luts) {
-    constexpr bool kKeepWords = ITERS <= 24;  // longer rows re-read their state words (L2 hits)
-    const int gpr = t.in_features >> 2;
+    constexpr bool kKeepWords = ITERS <= 16;  // longer rows re-read their state words (cache hits)
+    constexpr int kLast = ITERS - 1;
+    const uint32_t gpr = (uint32_t)t.in_features >> 2;
     const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    const uint32_t gi_last = (uint32_t)lane + kWave * kLast;
+    const bool last_live = gi_last < gpr;
+    const uint32_t gc_last = last_live ? gi_last : gpr - 1;
 
     float4 q[ITERS];
     uint32_t w[kKeepWords ? ITERS : 1];
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
-        const int gi = lane + kWave * j;
-        const int gc = gi < gpr ? gi : gpr - 1;
+        const uint32_t gc = j < kLast ? (uint32_t)lane + kWave * j : gc_last;
         q[j] = g_row[gc];
-        if (kKeepWords || WITH_GS) {
-            const uint32_t word = load_group_dword(s_row + 3 * gc);
-            if (kKeepWords) w[j] = word;
-        }
+        if (kKeepWords) w[j] = load_group_dword(s_row + 3u * gc);
     }
     RowAcc acc;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
-        const bool live = lane + kWave * j < gpr;
+        const bool live = j < kLast || last_live;
         // a masked group adds +0.0 (squares) and -+0.0 (0 * t): both leave the sums unchanged
         const float g[4] = {live ? q[j].x : 0.0f, live ? q[j].y : 0.0f, live ? q[j].z : 0.0f,
                             live ? q[j].w : 0.0f};
         uint32_t word = 0;
         if (WITH_GS) {
-            const int gi = lane + kWave * j;
-            word = kKeepWords ? w[j] : load_group_dword(s_row + 3 * (gi < gpr ? gi : gpr - 1));
+            const uint32_t gc = j < kLast ? (uint32_t)lane + kWave * j : gc_last;
+            word = kKeepWords ? w[j] : load_group_dword(s_row + 3u * gc);
         }
         accumulate<WITH_GS>(acc, g, word, a.cd);
     }
@@ -230,13 +249,12 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
     const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
-        const int gi = lane + kWave * j;
-        if (gi < gpr) {
-            const float g[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
-            const uint32_t word = kKeepWords ? w[j] : load_group_dword(s_row + 3 * gi);
-            const uint32_t nw = tick_group<true>(word, g, rc.tc, luts, row_elem + 4u * (uint32_t)gi);
-            store_group(s_row + 3 * gi, nw);
-        }
+        const uint32_t gi = (uint32_t)lane + kWave * j;
+        const uint32_t gc = j < kLast ? gi : gc_last;
+        const float g[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
+        const uint32_t word = kKeepWords ? w[j] : load_group_dword(s_row + 3u * gc);
+        const uint32_t nw = tick_group<true>(word, g, rc.tc, luts, row_elem + 4u * gi);
+        if (j < kLast || last_live) store_group(s_row + 3u * gi, nw);
     }
 }
 
@@ -261,7 +279,10 @@ __device__ __forceinline__ void update_row_streamed(const BatchArgs& a, const Up
 // Minimum waves per SIMD the compiler must leave room for: the tick arithmetic has long
 // dependent chains, so the row's registers are budgeted to keep 3-4 waves resident for short
 // rows and 2 for the longest.
-constexpr int min_waves(int iters) { return iters <= 8 ? 4 : (iters <= 16 ? 3 : 2); }
+#ifndef MCC_MIN_WAVES_16
+#define MCC_MIN_WAVES_16 3
+#endif
+constexpr int min_waves(int iters) { return iters <= 10 ? 4 : (iters <= 16 ? MCC_MIN_WAVES_16 : 2); }
 
 template <int ITERS, bool WITH_GS>
 __global__ __launch_bounds__(kThreads, min_waves(ITERS)) void update_rows_kernel(BatchArgs a) {
@@ -321,29 +342,36 @@ hipError_t launch_iters(hipStream_t stream, const BatchArgs& a) {
     return a.lr_scale != 0.0f ? launch_variant<ITERS, true>(stream, a) : launch_variant<ITERS, false>(stream, a);
 }
 
-// Register-resident variant that fits a row of `in_features` (0 = streamed fallback).
+// Row lengths (in units of 64 groups = 256 weights, rounded up) with a register-resident
+// variant: every length up to 4096 weights, and the longer rows of common model widths
+// (5120, 5632, 6144, 7168, 8192, 10240, 11008).  Anything else takes the streamed row.
+#ifdef MCC_EXPERIMENT_FEW_VARIANTS
+#define MCC_RESIDENT_ITERS(X) X(3) X(8) X(16) X(43)
+#else
+#define MCC_RESIDENT_ITERS(X) \
+    X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16) \
+    X(20) X(22) X(24) X(28) X(32) X(40) X(43)
+#endif
+
+// Register-resident variant of a row of `in_features` (0 = streamed fallback).
 int iters_class(const UpdateTensor& t) {
     const int iters = ((t.in_features >> 2) + kWave - 1) / kWave;
     const bool aligned = (reinterpret_cast<uintptr_t>(t.grad_w) & 15u) == 0;
     if (!aligned) return 0;
-    static const int classes[] = {1, 2, 3, 4, 8, 12, 16, 24, 32, 43};
-    for (int c : classes)
-        if (iters <= c) return c;
-    return 0;
+    switch (iters) {
+#define MCC_CASE(N) case N:
+        MCC_RESIDENT_ITERS(MCC_CASE)
+#undef MCC_CASE
+        return iters;
+        default: return 0;
+    }
 }
 
 hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
     switch (cls) {
-        case 1: return launch_iters<1>(stream, a);
-        case 2: return launch_iters<2>(stream, a);
-        case 3: return launch_iters<3>(stream, a);
-        case 4: return launch_iters<4>(stream, a);
-        case 8: return launch_iters<8>(stream, a);
-        case 12: return launch_iters<12>(stream, a);
-        case 16: return launch_iters<16>(stream, a);
-        case 24: return launch_iters<24>(stream, a);
-        case 32: return launch_iters<32>(stream, a);
-        case 43: return launch_iters<43>(stream, a);
+#define MCC_CASE(N) case N: return launch_iters<N>(stream, a);
+        MCC_RESIDENT_ITERS(MCC_CASE)
+#undef MCC_CASE
         default: return launch_iters<0>(stream, a);
     }
 }

@@ -3,7 +3,7 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmotifcl_amd.so")
+LIB_PATH = os.environ.get("MOTIFCL_AMD_LIB", os.path.join(HERE, "libmotifcl_amd.so"))
 
 _vp, _sz, _f, _u32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_uint32
 
