@@ -31,6 +31,15 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 C, LR, LR_SCALE, BETA, EPS = 11, 3e-3, 0.0, 0.9, 1e-3
 BYTES_PER_PARAM = 5.5          # 4 (read G) + 0.75 (read state) + 0.75 (write state)
 
+# HBM-side bytes per launch of the dominant kernels, measured offline with
+# `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` on this same command (scaled by a plain
+# 1 GiB copy; summaries and commands under profiles/).  They are reported, not re-measured
+# here, and only for the default workloads they were measured on.
+MEASURED_TRAFFIC_BYTES = {
+    "cfg4/gemm_tn_f32": 24.6e9,       # average over the 7 launches of a step (algorithmic 1.4 GB)
+    "cfg3/update_rows": 38.12e9,      # the batched call of a step (algorithmic 35.62 GB)
+}
+
 
 def layer_shapes(dim, hidden):
     """(out, in) of the seven linears of one block: Wq Wk Wv Wo, W1 W3, W2."""
@@ -134,7 +143,8 @@ def bench_fused(L, ops, name, steps, warmup):
                    "C": C, "lr": LR, "lr_scale": LR_SCALE, "rms_beta": BETA, "rms_eps": EPS},
         "roofline": {"bound": "mfma", "kernel": "gemm_tn_f32", "achieved": achieved,
                      "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_MFMA_F32_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_MFMA_F32_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name + "/gemm_tn_f32"),
                      "launches": gemm_n, "avg_launch_ms": gemm_ms / max(gemm_n, 1),
                      "algorithmic_flops_per_step": flops},
         "kernel_ms_per_step": {"gemm_tn_f32": gemm_ms / steps, "counter_update": upd_ms / steps},
@@ -185,7 +195,8 @@ def bench_update_only(L, ops, steps, warmup):
         # one timed region per call = the launches that cover all 224 tensors
         "roofline": {"bound": "hbm", "kernel": "update_rows_kernel", "achieved": achieved,
                      "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
-                     "traffic": None, "launches": upd_n, "avg_launch_ms": upd_ms / max(upd_n, 1),
+                     "traffic": MEASURED_TRAFFIC_BYTES["cfg3/update_rows"],
+                     "launches": upd_n, "avg_launch_ms": upd_ms / max(upd_n, 1),
                      "algorithmic_bytes_per_param": BYTES_PER_PARAM,
                      "algorithmic_bytes_per_launch": BYTES_PER_PARAM * params},
     }
@@ -241,6 +252,9 @@ def main():
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-update-only", action="store_true", help="skip the cfg3 update-only leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run one plain 1 GiB device copy (torch copy_), the known-size kernel that "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of one tensor for the CPU fused sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -255,6 +269,15 @@ def main():
     L = motifcl_amd.load()  # raises if the HIP library is missing: there is no fallback
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+
+    if args.traffic_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup)
     line = {
