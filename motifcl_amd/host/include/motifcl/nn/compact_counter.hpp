@@ -1,0 +1,56 @@
+// nn::CounterStateLinear with the public surface of
+// include/motifcl/nn/compact_counter.hpp:16-60 of MotifCL, implemented on the HIP library.
+#pragma once
+
+#include <cstdint>
+
+#include <motifcl/nn/module.hpp>
+#include <motifcl/runtime/backend.hpp>
+
+namespace motifcl::nn {
+
+// Ternary finite-state "counter" linear layer trained as a per-synapse automaton: the whole
+// trainable state is a packed 6-bit code per weight plus a per-row scale and a per-row RMS
+// second moment; the update is fused into backward.
+class CounterStateLinear : public Module {
+public:
+    CounterStateLinear(Backend& backend, int in_features, int out_features, int C = 11,
+                       float lr = 3e-3f, float lr_scale = 0.0f, float init_gain = 1.0f,
+                       float rms_beta = 0.9f, float rms_eps = 1e-3f, std::uint32_t seed = 12345u);
+
+    Tensor forward(const Tensor& x) override;
+    std::vector<Parameter*> parameters() override { return {}; }  // self-updating
+
+    Tensor decode_weight() const;                                      // dense [out, in] f32
+    void apply_update_seed(const Tensor& grad_w, std::uint32_t seed);  // update-only (dense grad_w)
+    void apply_update_backward(const Tensor& grad_out, const Tensor& x, std::uint32_t seed);  // fused
+    Tensor backward_input_from_state(const Tensor& grad_out) const;   // grad_x [N, in]
+    std::uint32_t next_seed() { return seed_++; }
+
+    void set_training(bool t) { training_ = t; }
+    bool training() const { return training_; }
+    void set_lr(float lr) { lr_ = lr; }
+    float lr() const { return lr_; }
+
+    int in_features() const { return in_; }
+    int out_features() const { return out_; }
+
+    // Persistent state (saved/restored as buffers, not optimizer-touched).
+    Tensor state;  // U8  [out * in/4 * 3]
+    Tensor scale;  // F32 [out]
+    Tensor v;      // F32 [out]
+
+private:
+    Backend* backend_ = nullptr;
+    int in_ = 0;
+    int out_ = 0;
+    int C_ = 11;
+    float lr_ = 3e-3f;
+    float lr_scale_ = 0.0f;
+    float rms_beta_ = 0.9f;
+    float rms_eps_ = 1e-3f;
+    std::uint32_t seed_ = 12345u;
+    bool training_ = true;
+};
+
+}  // namespace motifcl::nn

@@ -1,0 +1,146 @@
+// nn::CounterStateLinear on the HIP library.  Structure and ordering follow
+// src/nn/compact_counter.cpp of MotifCL: the constructor packs the initial state
+// (:55-85), the backward node computes grad_x from the pre-update state, then runs the fused
+// update under NoGradGuard, then propagates (:30-51), and forward attaches that node whenever
+// the layer is training, whether or not the input wants a gradient (:295-298).
+#include <motifcl/nn/compact_counter.hpp>
+
+#include <motifcl/autograd/node.hpp>
+#include <motifcl/core/error.hpp>
+
+#include <motifcl_amd.h>
+
+#include <cmath>
+#include <memory>
+#include <random>
+#include <string>
+#include <vector>
+
+namespace motifcl::nn {
+namespace {
+
+inline std::uint8_t cc_encode(int t, int c, int C) {
+    const int lv = 2 * C - 1;
+    return static_cast<std::uint8_t>((t + 1) * lv + (c + (C - 1)));
+}
+
+struct CounterBackwardNode : autograd::Node {
+    Tensor x;
+    CounterStateLinear* layer;
+    std::uint32_t seed;
+
+    CounterBackwardNode(Tensor x_, CounterStateLinear* l, std::uint32_t s) : x(std::move(x_)), layer(l), seed(s) {}
+
+    std::vector<Tensor> inputs() const override { return {x}; }
+
+    void backward(const Tensor& grad_out) override {
+        const bool need_gx = x.requires_grad();
+        Tensor grad_x;
+        if (need_gx) grad_x = layer->backward_input_from_state(grad_out);  // PRE-update state
+        {
+            autograd::NoGradGuard guard;
+            layer->apply_update_backward(grad_out, x, seed);
+        }
+        if (need_gx) x.backward(grad_x);
+    }
+};
+
+const float* f32(const Tensor& t) { return static_cast<const float*>(t.data()); }
+float* f32(Tensor& t) { return static_cast<float*>(t.data()); }
+
+}  // namespace
+
+CounterStateLinear::CounterStateLinear(Backend& backend, int in_features, int out_features, int C, float lr,
+                                       float lr_scale, float init_gain, float rms_beta, float rms_eps,
+                                       std::uint32_t seed)
+    : backend_(&backend), in_(in_features), out_(out_features), C_(C), lr_(lr), lr_scale_(lr_scale),
+      rms_beta_(rms_beta), rms_eps_(rms_eps), seed_(seed) {
+    MCL_CHECK(in_ > 0 && out_ > 0, "CounterStateLinear requires positive dimensions");
+    MCL_CHECK(C_ > 0 && 3 * (2 * C_ - 1) <= 64, "C too large for 6-bit packed state encoding");
+    MCL_CHECK(in_ % 4 == 0, "CounterStateLinear requires in_features divisible by 4 (6-bit packing)");
+
+    std::mt19937 rng(seed);
+    std::uniform_int_distribution<int> tern(-1, 1);
+    const int gpr = in_ / 4;
+    std::vector<std::uint8_t> st(static_cast<std::size_t>(out_) * gpr * 3);
+    for (int row = 0; row < out_; ++row)
+        for (int g = 0; g < gpr; ++g) {
+            std::uint32_t word = 0;
+            for (int k = 0; k < 4; ++k) word |= static_cast<std::uint32_t>(cc_encode(tern(rng), 0, C_)) << (6 * k);
+            std::uint8_t* p = st.data() + (static_cast<std::size_t>(row) * gpr + g) * 3;
+            p[0] = static_cast<std::uint8_t>(word & 0xFF);
+            p[1] = static_cast<std::uint8_t>((word >> 8) & 0xFF);
+            p[2] = static_cast<std::uint8_t>((word >> 16) & 0xFF);
+        }
+    state = Tensor::from_cpu(*backend_, {static_cast<int64_t>(out_) * gpr * 3}, DType::U8, st.data());
+
+    const float s0 = init_gain * std::sqrt(3.0f / (2.0f * static_cast<float>(in_)));
+    std::vector<float> sc(static_cast<std::size_t>(out_), s0);
+    std::vector<float> vv(static_cast<std::size_t>(out_), 0.0f);
+    scale = Tensor::from_cpu(*backend_, {out_}, DType::F32, sc.data());
+    v = Tensor::from_cpu(*backend_, {out_}, DType::F32, vv.data());
+}
+
+Tensor CounterStateLinear::decode_weight() const {
+    Tensor w = Tensor::empty(*backend_, {out_, in_}, DType::F32);
+    const int rc = mcc_compact_counter_decode_weight(
+        backend_->hip_stream(), static_cast<const std::uint8_t*>(state.data()), state.nbytes(), f32(scale),
+        scale.nbytes(), f32(w), w.nbytes(), static_cast<std::size_t>(in_), static_cast<std::size_t>(out_),
+        static_cast<std::size_t>(C_));
+    MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter decode_weight failed: ") + mcc_last_error());
+    return w;
+}
+
+void CounterStateLinear::apply_update_seed(const Tensor& grad_w, std::uint32_t seed) {
+    MCL_CHECK(grad_w.dtype() == DType::F32 && grad_w.numel() == static_cast<int64_t>(out_) * in_,
+              "apply_update_seed expects an f32 [out, in] gradient");
+    const int rc = mcc_compact_counter_apply_update_dense(
+        backend_->hip_stream(), static_cast<std::uint8_t*>(state.data()), state.nbytes(), f32(scale), scale.nbytes(),
+        f32(v), v.nbytes(), f32(grad_w), grad_w.nbytes(), static_cast<std::size_t>(C_), static_cast<std::size_t>(in_),
+        static_cast<std::size_t>(out_), lr_, lr_scale_, rms_beta_, rms_eps_, seed);
+    MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter update failed: ") + mcc_last_error());
+}
+
+void CounterStateLinear::apply_update_backward(const Tensor& grad_out, const Tensor& x, std::uint32_t seed) {
+    MCL_CHECK(x.ndim() == 2 && grad_out.ndim() == 2, "apply_update_backward expects rank-2 tensors");
+    const std::size_t N = static_cast<std::size_t>(x.shape()[0]);
+    const std::size_t ws = mcc_compact_counter_fused_workspace_nbytes(static_cast<std::size_t>(in_),
+                                                                     static_cast<std::size_t>(out_), N);
+    void* scratch = backend_->workspace(ws);
+    const int rc = mcc_compact_counter_apply_update_fused(
+        backend_->hip_stream(), static_cast<std::uint8_t*>(state.data()), state.nbytes(), f32(scale), scale.nbytes(),
+        f32(v), v.nbytes(), f32(grad_out), grad_out.nbytes(), f32(x), x.nbytes(), scratch, ws,
+        static_cast<std::size_t>(C_), static_cast<std::size_t>(in_), static_cast<std::size_t>(out_), N, lr_, lr_scale_,
+        rms_beta_, rms_eps_, seed);
+    MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter fused update failed: ") + mcc_last_error());
+}
+
+Tensor CounterStateLinear::backward_input_from_state(const Tensor& grad_out) const {
+    MCL_CHECK(grad_out.backend_ptr() == backend_, "CounterStateLinear backward_input backend mismatch");
+    const int N = static_cast<int>(grad_out.shape()[0]);
+    Tensor grad_x = Tensor::empty(*backend_, {N, in_}, DType::F32);
+    const int rc = mcc_compact_counter_backward_input_u8(
+        backend_->hip_stream(), static_cast<const std::uint8_t*>(state.data()), state.nbytes(), f32(scale),
+        scale.nbytes(), f32(grad_out), grad_out.nbytes(), f32(grad_x), grad_x.nbytes(), static_cast<std::size_t>(N),
+        static_cast<std::size_t>(in_), static_cast<std::size_t>(out_), static_cast<std::size_t>(C_));
+    MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter backward_input failed: ") + mcc_last_error());
+    return grad_x;
+}
+
+Tensor CounterStateLinear::forward(const Tensor& x) {
+    MCL_CHECK(x.dtype() == DType::F32 && x.ndim() == 2, "CounterStateLinear expects rank-2 f32 input");
+    MCL_CHECK(x.shape()[1] == in_, "CounterStateLinear input feature mismatch");
+    Tensor y = Tensor::empty(*backend_, {x.shape()[0], out_}, DType::F32);
+    const int rc = mcc_compact_counter_forward_u8(
+        backend_->hip_stream(), f32(x), x.nbytes(), static_cast<const std::uint8_t*>(state.data()), state.nbytes(),
+        f32(scale), scale.nbytes(), f32(y), y.nbytes(), static_cast<std::size_t>(x.shape()[0]),
+        static_cast<std::size_t>(in_), static_cast<std::size_t>(out_), static_cast<std::size_t>(C_));
+    MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter forward failed: ") + mcc_last_error());
+    if (autograd::is_enabled() && training_) {  // gate on training, not on x.requires_grad
+        y.set_requires_grad(true);
+        y._set_grad_fn(std::make_shared<CounterBackwardNode>(x, this, next_seed()));
+    }
+    return y;
+}
+
+}  // namespace motifcl::nn
