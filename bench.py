@@ -244,6 +244,39 @@ def cpu_baseline_dense(sample, min_seconds=4.0):
             "sample": "CPU oracle update-only on one [%d,%d] tensor, %d passes" % (n_out, n_in, reps)}
 
 
+def parity_leg(ops):
+    """Correctness gates reported beside the speed figures: BASELINE config 0 (one 288x288
+    tensor, 4096 tokens) on the GPU against the CPU oracle."""
+    import numpy as np
+    import torch
+    from oracle import counter_oracle as oracle
+    N, n_in, n_out = 4096, 288, 288
+    rng = np.random.default_rng(0)
+    state = oracle.pack_codes(rng.integers(0, 63, (n_out, n_in)).astype(np.uint8))
+    scale = np.full(n_out, math.sqrt(3.0 / (2.0 * n_in)), dtype=np.float32)
+    v = np.zeros(n_out, dtype=np.float32)
+    x = rng.standard_normal((N, n_in)).astype(np.float32)
+    dy = (rng.standard_normal((N, n_out)) * 0.01).astype(np.float32)
+    d = [torch.from_numpy(a).cuda() for a in (state, scale, v)]
+    ws = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, N), dtype=torch.uint8, device="cuda")
+    ops.apply_update_fused(*d, torch.from_numpy(dy).cuda(), torch.from_numpy(x).cuda(), ws,
+                           C, LR, LR_SCALE, BETA, EPS, 12345)
+    torch.cuda.synchronize()
+    g_gpu = ws.view(torch.float32)[: n_out * n_in].view(n_out, n_in).cpu().numpy()
+    e_state, e_scale, e_v, g_seq = oracle.update_fused(state, scale, v, dy, x, C, LR, LR_SCALE, BETA, EPS, 12345)
+    x_state, x_scale, x_v = oracle.update_dense(state, scale, v, g_gpu, C, LR, LR_SCALE, BETA, EPS, 12345)
+    got = [t.cpu().numpy() for t in d]
+    return {
+        "workload": "cfg0: 288x288, 4096 tokens, one fused update, GPU vs CPU oracle",
+        "state_scale_v_bit_exact_given_gpu_gradient": bool(
+            np.array_equal(got[0], x_state) and np.array_equal(got[1], x_scale) and np.array_equal(got[2], x_v)),
+        "max_abs_dG_over_max_abs_G_vs_sequential_sum": float(np.abs(g_gpu - g_seq).max() / np.abs(g_seq).max()),
+        "counter_flip_mismatch_fraction_vs_sequential_sum": float(
+            (oracle.unpack_codes(got[0]) != oracle.unpack_codes(e_state)).mean()),
+        "counters_changed_fraction": float((oracle.unpack_codes(got[0]) != oracle.unpack_codes(state)).mean()),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -291,6 +324,7 @@ def main():
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_fused(fused_sample, tokens, args.cpu_rows)
+        line["parity"] = parity_leg(ops)
     del fused_sample
     torch.cuda.empty_cache()
     if not args.no_update_only:

@@ -187,12 +187,13 @@ __device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], con
 // Tick pass over a row re-read from memory with byte-granular state access: the fallback for
 // rows of any length and alignment, and for rows that need the plain division.
 __device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, int lane, const TickConsts& tc,
-                                               const Luts& l) {
+                                               const Luts& l, int group_begin = 0, int group_end = 0x7fffffff) {
     const int gpr = t.in_features >> 2;
+    const int g_end = group_end < gpr ? group_end : gpr;
     const float* g_row = t.grad_w + (size_t)row * t.in_features;
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
     const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
-    for (int gi = lane; gi < gpr; gi += kWave) {
+    for (int gi = group_begin + lane; gi < g_end; gi += kWave) {
         float g[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) g[k] = g_row[4 * gi + k];
@@ -311,6 +312,135 @@ __global__ __launch_bounds__(kThreads, min_waves(ITERS)) void update_rows_kernel
     }
 }
 
+// ---------------------------------------------------------------------------
+// Long rows: W cooperating waves per row.  Wave w keeps iterations [w*J, (w+1)*J) of the row in
+// its registers, so a row of up to 64*J*W groups is register-resident with J*5 instead of
+// ITERS*5 row registers per lane, and three or four waves per SIMD still fit.  The reference's
+// per-lane partial sums are sequential in the iteration index, so the running sums are handed
+// from wave to wave through LDS (W-1 barriers); the last wave owns the tree, the row epilogue
+// and the commit, and publishes the tick constants for everybody's share of the tick pass.
+// ---------------------------------------------------------------------------
+struct SplitShared {
+    Luts luts;
+    float part_sq[kWave];
+    float part_gs[kWave];
+    uint32_t part_key[kWave];
+    TickConsts tc;
+    int fast_div;
+};
+
+constexpr int min_waves_split(int j) { return j <= 6 ? 4 : 3; }
+
+template <int J, int W, bool WITH_GS>
+__global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_split_kernel(BatchArgs a) {
+    __shared__ SplitShared sh;
+    build_luts(sh.luts, a.cd, a.geom);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int ti = 0;
+    for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
+        const int grow = __builtin_amdgcn_readfirstlane(grow_v);
+        ti = __builtin_amdgcn_readfirstlane(ti);
+        while (grow >= a.t[ti].row_start + a.t[ti].out_features) ++ti;  // monotonic
+        ti = __builtin_amdgcn_readfirstlane(ti);
+        const UpdateTensor t = a.t[ti];
+        const int row = grow - t.row_start;
+        if (row == t.out_features - 1) {
+            // byte-granular path for the tensor's last row, by wave 0; the others only keep the
+            // workgroup's barrier count in step (finish_row synchronises twice)
+            if (w == 0) {
+                update_row_streamed<WITH_GS>(a, t, row, lane, sh.luts);
+            } else {
+                __syncthreads();
+                __syncthreads();
+            }
+            continue;
+        }
+        const uint32_t gpr = (uint32_t)t.in_features >> 2;
+        const int iters = (int)((gpr + kWave - 1) / kWave);
+        const int j0 = w * J;
+        const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
+        uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+
+        float4 q[J];
+        uint32_t words[J];
+#pragma unroll
+        for (int jj = 0; jj < J; ++jj) {
+            const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
+            const uint32_t gc = gi < gpr ? gi : gpr - 1;
+            q[jj] = g_row[gc];
+            words[jj] = load_group_dword(s_row + 3u * gc);
+        }
+        // running sums travel wave 0 -> 1 -> ... -> W-1 in iteration order
+        RowAcc acc;
+#pragma unroll
+        for (int step = 0; step < W; ++step) {
+            if (w == step) {
+                if (step > 0) {
+                    acc.g_sq = sh.part_sq[lane];
+                    acc.grad_s = sh.part_gs[lane];
+                    acc.min_key = sh.part_key[lane];
+                }
+#pragma unroll
+                for (int jj = 0; jj < J; ++jj) {
+                    const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+                    const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
+                                        live ? q[jj].w : 0.0f};
+                    accumulate<WITH_GS>(acc, g, words[jj], a.cd);
+                }
+                if (step < W - 1) {
+                    sh.part_sq[lane] = acc.g_sq;
+                    sh.part_gs[lane] = acc.grad_s;
+                    sh.part_key[lane] = acc.min_key;
+                }
+            }
+            __syncthreads();
+        }
+        if (w == W - 1) {
+            const float g_sq = tree_sum(acc.g_sq, lane);
+            const float grad_s = WITH_GS ? tree_sum(acc.grad_s, lane) : 0.0f;
+            const uint32_t min_key = wave_min(acc.min_key, lane);
+            const float s_old = t.scale[row];
+            const float v_old = t.v[row];
+            const RowStats rs = finish_row_stats(g_sq, grad_s, v_old, s_old, t.in_features, a.lr_scale,
+                                                 a.rms_beta, a.rms_eps);
+            sh.luts.c_reb[lane] = c_reb_entry((uint32_t)lane, a.cd, s_old / rs.scale_new);
+            if (lane == 0) {
+                t.v[row] = rs.v_new;
+                t.scale[row] = rs.scale_new;
+                TickConsts tc;
+                tc.dn = rs.denom;
+                tc.r = 1.0f / rs.denom;
+                tc.k = a.cd.Cf / rs.scale_new;
+                tc.neg_lr = -t.lr;
+                tc.neg_lim_neg = -(float)a.geom.lim_neg;
+                tc.lim_pos = (float)a.geom.lim_pos;
+                tc.seed = t.seed;
+                tc.shift = a.geom.shift;
+                sh.tc = tc;
+                sh.fast_div = row_takes_fast_division(rs.denom, g_sq, min_key) ? 1 : 0;
+            }
+        }
+        __syncthreads();
+        const TickConsts tc = sh.tc;
+        const bool fast = __builtin_amdgcn_readfirstlane(sh.fast_div) != 0;
+        if (!fast) {
+            apply_streamed(t, row, lane, tc, sh.luts, j0 * kWave, (j0 + J) * kWave);
+            continue;
+        }
+        const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
+#pragma unroll
+        for (int jj = 0; jj < J; ++jj) {
+            if (j0 + jj < iters) {  // wave-uniform
+                const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
+                const float g[4] = {q[jj].x, q[jj].y, q[jj].z, q[jj].w};
+                const uint32_t nw = tick_group<true>(words[jj], g, tc, sh.luts, row_elem + 4u * gi);
+                if (gi < gpr) store_group(s_row + 3u * gi, nw);
+            }
+        }
+    }
+}
+
 int device_cu_count() {
     static int cus = [] {
         int dev = 0, n = 0;
@@ -337,34 +467,64 @@ hipError_t launch_variant(hipStream_t stream, const BatchArgs& a) {
     return hipGetLastError();
 }
 
+template <int J, int W, bool WITH_GS>
+hipError_t launch_split_variant(hipStream_t stream, const BatchArgs& a) {
+    static int blocks_per_cu = [] {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_split_kernel<J, W, WITH_GS>, kWave * W, 0) !=
+                hipSuccess || n <= 0)
+            n = 1;
+        return n;
+    }();
+    const int resident = device_cu_count() * blocks_per_cu;
+    const dim3 grid(a.total_rows < resident ? a.total_rows : resident);
+    hipLaunchKernelGGL((update_rows_split_kernel<J, W, WITH_GS>), grid, dim3(kWave * W), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <int J, int W>
+hipError_t launch_split(hipStream_t stream, const BatchArgs& a) {
+    return a.lr_scale != 0.0f ? launch_split_variant<J, W, true>(stream, a) : launch_split_variant<J, W, false>(stream, a);
+}
+
 template <int ITERS>
 hipError_t launch_iters(hipStream_t stream, const BatchArgs& a) {
     return a.lr_scale != 0.0f ? launch_variant<ITERS, true>(stream, a) : launch_variant<ITERS, false>(stream, a);
 }
 
-// Row lengths (in units of 64 groups = 256 weights, rounded up) with a register-resident
-// variant: every length up to 4096 weights, and the longer rows of common model widths
-// (5120, 5632, 6144, 7168, 8192, 10240, 11008).  Anything else takes the streamed row.
+// Row lengths (in units of 64 groups = 256 weights, rounded up) with a one-wave
+// register-resident variant: every length up to 4096 weights.  Longer rows, up to 22528
+// weights, are shared by four or eight waves; anything beyond takes the streamed row.
 #ifdef MCC_EXPERIMENT_FEW_VARIANTS
-#define MCC_RESIDENT_ITERS(X) X(3) X(8) X(16) X(43)
+#define MCC_RESIDENT_ITERS(X) X(3) X(8) X(16)
 #else
 #define MCC_RESIDENT_ITERS(X) \
-    X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16) \
-    X(20) X(22) X(24) X(28) X(32) X(40) X(43)
+    X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16)
 #endif
+
+// Classes of the split kernel are encoded as 1000 + 10*J + W.
+constexpr int split_class(int j, int w) { return 1000 + 10 * j + w; }
 
 // Register-resident variant of a row of `in_features` (0 = streamed fallback).
 int iters_class(const UpdateTensor& t) {
     const int iters = ((t.in_features >> 2) + kWave - 1) / kWave;
     const bool aligned = (reinterpret_cast<uintptr_t>(t.grad_w) & 15u) == 0;
     if (!aligned) return 0;
+#ifdef MCC_EXPERIMENT_SPLIT16
+    if (iters > 8 && iters <= 16) return split_class(8, 2);
+#endif
     switch (iters) {
 #define MCC_CASE(N) case N:
         MCC_RESIDENT_ITERS(MCC_CASE)
 #undef MCC_CASE
         return iters;
-        default: return 0;
+        default: break;
     }
+    if (iters > 16 && iters <= 24) return split_class(6, 4);
+    if (iters > 24 && iters <= 32) return split_class(8, 4);
+    if (iters > 32 && iters <= 44) return split_class(11, 4);
+    if (iters > 44 && iters <= 88) return split_class(11, 8);
+    return 0;
 }
 
 hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
@@ -372,6 +532,13 @@ hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
 #define MCC_CASE(N) case N: return launch_iters<N>(stream, a);
         MCC_RESIDENT_ITERS(MCC_CASE)
 #undef MCC_CASE
+#ifdef MCC_EXPERIMENT_SPLIT16
+        case split_class(8, 2): return launch_split<8, 2>(stream, a);
+#endif
+        case split_class(6, 4): return launch_split<6, 4>(stream, a);
+        case split_class(8, 4): return launch_split<8, 4>(stream, a);
+        case split_class(11, 4): return launch_split<11, 4>(stream, a);
+        case split_class(11, 8): return launch_split<11, 8>(stream, a);
         default: return launch_iters<0>(stream, a);
     }
 }
