@@ -20,15 +20,20 @@
 
 namespace mcc {
 
-// lowbias32 (kernels/compact_counter.cl:17-21)
-MCC_HD uint32_t hash_u32(uint32_t x) {
-    x ^= x >> 16;
+// lowbias32 (kernels/compact_counter.cl:17-21), split after its first xor-shift: the four
+// elements of a packed group have indices e, e+1, e+2, e+3 with e a multiple of 4, and
+// (e + k) ^ ((e + k) >> 16) == (e ^ (e >> 16)) ^ k for k < 4, so the first step is shared.
+MCC_HD uint32_t hash_first(uint32_t x) { return x ^ (x >> 16); }
+
+MCC_HD uint32_t hash_rest(uint32_t x) {
     x *= 0x7feb352du;
     x ^= x >> 15;
     x *= 0x846ca68bu;
     x ^= x >> 16;
     return x;
 }
+
+MCC_HD uint32_t hash_u32(uint32_t x) { return hash_rest(hash_first(x)); }
 
 // 24-bit word of one packed group -> code k (kernels/compact_counter.cl:25-31)
 MCC_HD uint32_t code_of(uint32_t word, int k) { return (word >> (6 * k)) & 0x3fu; }
@@ -59,7 +64,7 @@ MCC_HD int code_q(uint32_t code, const Codec& cd) { return (int)((code * cd.magi
 // q = t + 1 (from the old code), total = floor(val) + [rnd < frac], and C
 // (kernels/compact_counter.cl:126-136).  It is tabulated once per kernel launch:
 //
-//   fin[(total + lim_neg) << shift | q] = new 6-bit code
+//   fin[q * width + (total + lim_neg)] = new 6-bit code
 //
 // Range of `total` that can matter: with t = q - 1 in [-1, rows - 2]
 // (rows = 63/lv + 1 distinct q values) the ternary value saturates upward as
@@ -72,19 +77,16 @@ MCC_HD int code_q(uint32_t code, const Codec& cd) { return (int)((code * cd.magi
 // ---------------------------------------------------------------------------
 struct LutGeom {
     int rows;      // distinct q = code / lv values
-    int shift;     // log2 of the q-stride of the table (power of two >= rows)
     int lim_neg;   // clamp of floor(val) below, as a positive number
     int lim_pos;   // clamp of floor(val) above
     int width;     // number of distinct totals: lim_neg + lim_pos + 2
 };
 
-constexpr int kLutFinMaxBytes = 4480;  // C = 1: width 70 << shift 6
+constexpr int kLutFinMaxBytes = 4480;  // C = 1: 64 rows x width 70
 
 MCC_HD LutGeom lut_geom(const Codec& cd) {
     LutGeom g;
     g.rows = 63 / cd.lv + 1;
-    g.shift = 0;
-    while ((1 << g.shift) < g.rows) ++g.shift;
     g.lim_neg = g.rows * cd.C + 1;
     g.lim_pos = 3 * cd.C;
     g.width = g.lim_neg + g.lim_pos + 2;
@@ -104,7 +106,8 @@ MCC_HD uint32_t fin_entry(int total, int q, const Codec& cd) {
 }
 
 // Decode tables, indexed by the 6-bit code:
-//   q_off[code] = code / lv + (lim_neg << shift)   (t + 1, pre-biased for the fin index)
+//   q_off[code] = (code / lv) * width + lim_neg     (row of the fin table, pre-biased so that
+//                                                     fin index = q_off + total)
 //   c_reb[code] = (float)(code % lv - (C-1)) * (s_old / s_new)
 // c_reb is the rebased residual counter of kernels/compact_counter.cl:124; it depends on the
 // row through the scale ratio only, so it is tabulated once per row (64 products) instead of
@@ -114,17 +117,19 @@ MCC_HD int code_c(uint32_t code, const Codec& cd) {
 }
 
 MCC_HD int q_off_entry(uint32_t code, const Codec& cd, const LutGeom& g) {
-    return code_q(code, cd) + (g.lim_neg << g.shift);
+    return code_q(code, cd) * g.width + g.lim_neg;
 }
 
 MCC_HD float c_reb_entry(uint32_t code, const Codec& cd, float ratio) {
     return (float)code_c(code, cd) * ratio;
 }
 
+MCC_HD int fin_size(const LutGeom& g) { return g.rows * g.width; }
+
 MCC_HD void fill_fin_entry(int idx, const Codec& cd, const LutGeom& g, uint8_t* fin) {
-    const int til = idx >> g.shift;
-    const int q = idx & ((1 << g.shift) - 1);
-    fin[idx] = q < g.rows ? (uint8_t)fin_entry(til - g.lim_neg, q, cd) : (uint8_t)0;
+    const int q = idx / g.width;
+    const int til = idx - q * g.width;
+    fin[idx] = (uint8_t)fin_entry(til - g.lim_neg, q, cd);
 }
 
 // Division by the per-row denominator, gw / dn, without a per-element reciprocal: with
@@ -179,26 +184,27 @@ struct TickConsts {
     float k;          // Cf / s_new
     float neg_lr;     // -lr
     float neg_lim_neg, lim_pos;  // clamp of floor(val), as floats
+    float two_m24;               // 2^-24 (kept in a register: see the kernel)
     uint32_t seed;
-    int shift;
 };
 
 // One stochastic-rounding tick (kernels/compact_counter.cl:120-136).
 //   code : current 6-bit code           gw   : weight gradient of this element
-//   elem : row*in + i (the RNG index)
-//   c_reb, q_off : the decode tables above;  fin : the (total, q) -> code table
+//   elem_x : hash_first(row*in + i), the RNG index after the first xor-shift
+//   c_reb, q_off : the decode tables above;  fin : the (q, total) -> code table
 // Returns the new 6-bit code.
 template <bool FAST_DIV, typename CReb, typename QOff, typename Fin>
-MCC_HD uint32_t tick_code(uint32_t code, float gw, const TickConsts& tc, uint32_t elem,
+MCC_HD uint32_t tick_code(uint32_t code, float gw, const TickConsts& tc, uint32_t elem_x,
                           CReb c_reb, QOff q_off, Fin fin) {
     const float tick = (tc.neg_lr * div_by_row<FAST_DIV>(gw, tc.dn, tc.r)) * tc.k;
     const float val = c_reb[code] + tick;
     const float f = floorf(val);
     const float frac = val - f;
-    const uint32_t h = hash_u32(tc.seed ^ hash_u32(elem));
-    const float rnd = (float)(h & 0x00ffffffu) * (1.0f / 16777216.0f);
-    const int til = (int)clamp_f(f, tc.neg_lim_neg, tc.lim_pos) + (rnd < frac ? 1 : 0);
-    return fin[((uint32_t)til << tc.shift) + (uint32_t)q_off[code]];
+    const uint32_t h = hash_u32(tc.seed ^ hash_rest(elem_x));
+    const float rnd = (float)(h & 0x00ffffffu) * tc.two_m24;
+    // q_off + floor + [rnd < frac]: one add-with-carry on the GPU
+    const int idx = q_off[code] + (int)clamp_f(f, tc.neg_lim_neg, tc.lim_pos) + (rnd < frac ? 1 : 0);
+    return fin[idx];
 }
 
 // Row statistics epilogue (kernels/compact_counter.cl:92-99), given the tree

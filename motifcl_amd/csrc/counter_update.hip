@@ -55,7 +55,7 @@ struct Luts {
 
 __device__ __forceinline__ void build_luts(Luts& l, const Codec& cd, const LutGeom& geom) {
     for (int i = threadIdx.x; i < 64; i += blockDim.x) l.q_off[i] = q_off_entry((uint32_t)i, cd, geom);
-    const int n = geom.width << geom.shift;
+    const int n = fin_size(geom);
     for (int i = threadIdx.x; i < n; i += blockDim.x) fill_fin_entry(i, cd, geom, l.fin);
     __syncthreads();
 }
@@ -66,9 +66,11 @@ __device__ __forceinline__ uint32_t load_group(const uint8_t* p) {
 }
 
 __device__ __forceinline__ void store_group(uint8_t* p, uint32_t w) {
-    p[0] = (uint8_t)(w & 0xffu);
-    p[1] = (uint8_t)((w >> 8) & 0xffu);
-    p[2] = (uint8_t)((w >> 16) & 0xffu);
+    // a 2-byte and a 1-byte store straight out of the word's register (global memory takes the
+    // unaligned 2-byte store); no repacking
+    const uint16_t lo = (uint16_t)w;
+    __builtin_memcpy(p, &lo, 2);
+    p[2] = (uint8_t)(w >> 16);
 }
 
 // One group's 24-bit word fetched with a single 4-byte load (global memory takes unaligned
@@ -87,14 +89,19 @@ struct RowAcc {
     uint32_t min_key = 0xffffffffu;
 };
 
+__device__ __forceinline__ uint32_t umin3(uint32_t a, uint32_t b, uint32_t c) {
+    const uint32_t ab = b < a ? b : a;
+    return c < ab ? c : ab;  // one v_min3_u32
+}
+
 template <bool WITH_GS>
 __device__ __forceinline__ void accumulate(RowAcc& acc, const float g[4], uint32_t w, const Codec& cd) {
+    acc.min_key = umin3(acc.min_key, range_key(g[0]), range_key(g[1]));
+    acc.min_key = umin3(acc.min_key, range_key(g[2]), range_key(g[3]));
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const float sq = g[k] * g[k];
         acc.g_sq = acc.g_sq + sq;
-        const uint32_t key = range_key(g[k]);
-        acc.min_key = key < acc.min_key ? key : acc.min_key;
         if (WITH_GS) {
             const int t = code_q(code_of(w, k), cd) - 1;
             const float gt = g[k] * (float)t;
@@ -167,7 +174,10 @@ __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTen
     rc.tc.neg_lim_neg = -(float)a.geom.lim_neg;
     rc.tc.lim_pos = (float)a.geom.lim_pos;
     rc.tc.seed = t.seed;
-    rc.tc.shift = a.geom.shift;
+    rc.tc.two_m24 = 1.0f / 16777216.0f;
+    // v_mul_f32 issues at twice the rate when both operands are VGPRs: keep the per-row
+    // multipliers out of scalar registers and literals
+    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24));
     rc.fast_div = __builtin_amdgcn_readfirstlane(row_takes_fast_division(rs.denom, g_sq, min_key) ? 1 : 0) != 0;
     return rc;
 }
@@ -176,9 +186,10 @@ template <bool FAST_DIV>
 __device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], const TickConsts& tc,
                                                const Luts& l, uint32_t elem0) {
     uint32_t nw = 0;
+    const uint32_t x0 = hash_first(elem0);  // elem0 is a multiple of 4: elements k share it up to ^k
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const uint32_t nc = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, elem0 + (uint32_t)k, l.c_reb, l.q_off, l.fin);
+        const uint32_t nc = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, x0 ^ (uint32_t)k, l.c_reb, l.q_off, l.fin);
         nw |= nc << (6 * k);
     }
     return nw;
@@ -416,13 +427,14 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
                 tc.neg_lim_neg = -(float)a.geom.lim_neg;
                 tc.lim_pos = (float)a.geom.lim_pos;
                 tc.seed = t.seed;
-                tc.shift = a.geom.shift;
+                tc.two_m24 = 1.0f / 16777216.0f;
                 sh.tc = tc;
                 sh.fast_div = row_takes_fast_division(rs.denom, g_sq, min_key) ? 1 : 0;
             }
         }
         __syncthreads();
-        const TickConsts tc = sh.tc;
+        TickConsts tc = sh.tc;
+        asm volatile("" : "+v"(tc.neg_lr), "+v"(tc.k), "+v"(tc.two_m24));  // VGPR multipliers
         const bool fast = __builtin_amdgcn_readfirstlane(sh.fast_div) != 0;
         if (!fast) {
             apply_streamed(t, row, lane, tc, sh.luts, j0 * kWave, (j0 + J) * kWave);

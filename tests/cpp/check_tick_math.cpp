@@ -6,6 +6,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <initializer_list>
 #include <vector>
 
 #include "../../motifcl_amd/csrc/counter_math.hpp"
@@ -27,12 +28,12 @@ int main(int argc, char** argv) {
     for (int C = 1; C <= 11; ++C) {
         const mcc::Codec cd = mcc::make_codec(C);
         const mcc::LutGeom g = mcc::lut_geom(cd);
-        if ((g.width << g.shift) > mcc::kLutFinMaxBytes) { std::printf("LUT too large for C=%d\n", C); return 2; }
-        std::vector<uint8_t> fin(g.width << g.shift);
+        if (mcc::fin_size(g) > mcc::kLutFinMaxBytes) { std::printf("LUT too large for C=%d\n", C); return 2; }
+        std::vector<uint8_t> fin(mcc::fin_size(g));
         std::vector<int> q_off(64);
         std::vector<float> c_reb(64);
         for (uint32_t code = 0; code < 64; ++code) q_off[code] = mcc::q_off_entry(code, cd, g);
-        for (int i = 0; i < (g.width << g.shift); ++i) mcc::fill_fin_entry(i, cd, g, fin.data());
+        for (int i = 0; i < mcc::fin_size(g); ++i) mcc::fill_fin_entry(i, cd, g, fin.data());
         // (code * magic) >> 16 == code / lv
         for (uint32_t code = 0; code < 64; ++code)
             if (mcc::code_q(code, cd) != (int)code / cd.lv) { std::printf("magic division fails C=%d code=%u\n", C, code); return 2; }
@@ -40,7 +41,7 @@ int main(int argc, char** argv) {
             mcc::TickConsts tc;
             tc.dn = dn; tc.r = 1.0f / dn; tc.k = cd.Cf / s_new; tc.neg_lr = -lr;
             tc.neg_lim_neg = -(float)g.lim_neg; tc.lim_pos = (float)g.lim_pos;
-            tc.seed = seed; tc.shift = g.shift;
+            tc.seed = seed; tc.two_m24 = 1.0f / 16777216.0f;
             for (uint32_t code = 0; code < 64; ++code) c_reb[code] = mcc::c_reb_entry(code, cd, s_old / s_new);
             return tc;
         };
@@ -73,8 +74,8 @@ int main(int argc, char** argv) {
                                                            mcc::range_key(gw));
             n_fast += fast;
             const uint32_t got = fast
-                ? mcc::tick_code<true>((uint32_t)code, gw, tc, elem, c_reb.data(), q_off.data(), fin.data())
-                : mcc::tick_code<false>((uint32_t)code, gw, tc, elem, c_reb.data(), q_off.data(), fin.data());
+                ? mcc::tick_code<true>((uint32_t)code, gw, tc, mcc::hash_first(elem), c_reb.data(), q_off.data(), fin.data())
+                : mcc::tick_code<false>((uint32_t)code, gw, tc, mcc::hash_first(elem), c_reb.data(), q_off.data(), fin.data());
             const int exp = oracle_tick_code(code, gw, s_old, s_new, dn, C, lr, seed, elem);
             ++checked;
             if ((int)got != exp) {
@@ -89,12 +90,21 @@ int main(int argc, char** argv) {
             for (int gi = -4 * 64; gi <= 4 * 64; ++gi) {
                 const float s = (float)C / 4.0f;
                 const mcc::TickConsts tc = make_tc(64.0f, s, s, 16.0f, 1u);
-                const uint32_t got = mcc::tick_code<true>((uint32_t)code, (float)gi, tc, 2u, c_reb.data(), q_off.data(), fin.data());
+                const uint32_t got = mcc::tick_code<true>((uint32_t)code, (float)gi, tc, mcc::hash_first(2u), c_reb.data(), q_off.data(), fin.data());
                 const int exp = oracle_tick_code(code, (float)gi, s, s, 64.0f, C, 16.0f, 1u, 2u);
                 ++checked;
                 if ((int)got != exp) { if (mismatches < 10) std::printf("TABLE MISMATCH C=%d code=%d g=%d got=%u exp=%d\n", C, code, gi, got, exp); ++mismatches; }
             }
     }
+    // shared first hash step: (e + k) ^ ((e + k) >> 16) == (e ^ (e >> 16)) ^ k for e % 4 == 0
+    for (long it = 0; it < 4000000; ++it) {
+        const uint32_t e = (uint32_t)next_u64() & ~3u;
+        for (uint32_t k = 0; k < 4; ++k)
+            if (mcc::hash_first(e + k) != (mcc::hash_first(e) ^ k)) { std::printf("hash_first sharing fails at %u+%u\n", e, k); return 2; }
+    }
+    for (uint32_t e : {0xfffcu, 0x1fffcu, 0xfffffffcu, 0x7ffffffcu, 0u})
+        for (uint32_t k = 0; k < 4; ++k)
+            if (mcc::hash_first(e + k) != (mcc::hash_first(e) ^ k)) { std::printf("hash_first sharing fails at %u+%u\n", e, k); return 2; }
     std::printf("checked %ld ticks (%ld through the reciprocal division), %ld mismatches\n", checked, n_fast, mismatches);
     return mismatches == 0 ? 0 : 1;
 }
