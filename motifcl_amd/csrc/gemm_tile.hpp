@@ -1,0 +1,144 @@
+// Main loop of the fp32 MFMA contraction c[m,n] = sum_k a[k,m] * b[k,n], shared by the plain
+// contraction kernel and the strip-fused update kernel.
+//
+// Both operands are stored token-major, which is exactly the operand shape of
+// v_mfma_f32_32x32x2_f32: lane l supplies a[k0 + l/32][m0 + l%32] and b[k0 + l/32][n0 + l%32],
+// i.e. 32 consecutive floats of one token row per half-wave.  Slabs of kBK tokens are staged
+// into LDS in their HBM orientation ([k][m] and [k][n]) with 16-byte loads and read back with
+// conflict-free 4-byte reads; no transpose is needed.  A workgroup of 4 waves (2x2) owns a
+// BM x BN tile; each wave owns (BM/2) x (BN/2) as 32x32 MFMA tiles whose accumulators stay in
+// registers for the whole K loop.  The next slab is fetched from HBM into registers while the
+// current one is multiplied.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+
+namespace mcc {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kGemmThreads = 256;
+constexpr int kBK = 16;  // tokens per LDS slab
+
+template <int BM, int BN>
+struct TileCfg {
+    static constexpr int kWaveM = BM / 2;        // rows of c per wave
+    static constexpr int kWaveN = BN / 2;        // cols of c per wave
+    static constexpr int kTilesM = kWaveM / 32;  // 32x32 MFMA tiles per wave along m
+    static constexpr int kTilesN = kWaveN / 32;
+    static constexpr int kLdA = BM + 4;  // padded LDS row strides (floats)
+    static constexpr int kLdB = BN + 4;
+    static constexpr int kA4 = kBK * BM / 4 / kGemmThreads;  // float4 loads per thread per slab
+    static constexpr int kB4 = kBK * BN / 4 / kGemmThreads;
+    static constexpr int kLdsFloats = kBK * (kLdA + kLdB);
+};
+
+// One slab row segment of 4 floats, zero-filled outside the matrix.
+template <bool VEC>
+__device__ __forceinline__ float4 load4(const float* __restrict__ base, int row, int col, int rows, int cols) {
+    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (row >= rows) return r;
+    const float* p = base + (size_t)row * cols + col;
+    if (VEC) {
+        if (col + 3 < cols) return *reinterpret_cast<const float4*>(p);
+    }
+    if (col + 0 < cols) r.x = p[0];
+    if (col + 1 < cols) r.y = p[1];
+    if (col + 2 < cols) r.z = p[2];
+    if (col + 3 < cols) r.w = p[3];
+    return r;
+}
+
+// Position of the calling thread inside its workgroup's tile.
+struct TilePos {
+    int tid, l32, half, wm0, wn0;
+};
+
+template <int BM, int BN>
+__device__ __forceinline__ TilePos tile_pos() {
+    using Cfg = TileCfg<BM, BN>;
+    TilePos p;
+    p.tid = threadIdx.x;
+    const int lane = p.tid & 63, wave = p.tid >> 6;
+    p.l32 = lane & 31;
+    p.half = lane >> 5;
+    p.wm0 = (wave >> 1) * Cfg::kWaveM;
+    p.wn0 = (wave & 1) * Cfg::kWaveN;
+    return p;
+}
+
+// Accumulates the BM x BN tile at (m0, n0) over all K tokens into acc (zeroed here).  lds holds
+// TileCfg::kLdsFloats floats.  Ends with a barrier, so lds may be reused right after.
+// Accumulator layout (v_mfma_f32_32x32x2_f32): acc[i][j][r] is row
+// wm0 + 32 i + 8 (r/4) + 4 half + r%4 and column wn0 + 32 j + l32 of the tile.
+template <int BM, int BN, bool VEC_A, bool VEC_B>
+__device__ __forceinline__ void gemm_tile_mainloop(const float* __restrict__ a, const float* __restrict__ b,
+                                                   int K, int M, int N, int m0, int n0, const TilePos& tp,
+                                                   float* lds,
+                                                   floatx16 (&acc)[TileCfg<BM, BN>::kTilesM][TileCfg<BM, BN>::kTilesN]) {
+    using Cfg = TileCfg<BM, BN>;
+    float* lds_a = lds;
+    float* lds_b = lds + kBK * Cfg::kLdA;
+#pragma unroll
+    for (int i = 0; i < Cfg::kTilesM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::kTilesN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    float4 ra[Cfg::kA4], rb[Cfg::kB4];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int p = 0; p < Cfg::kA4; ++p) {
+            const int idx = tp.tid + kGemmThreads * p;
+            const int row = idx / (BM / 4), c4 = idx % (BM / 4);
+            ra[p] = load4<VEC_A>(a, k0 + row, m0 + 4 * c4, K, M);
+        }
+#pragma unroll
+        for (int p = 0; p < Cfg::kB4; ++p) {
+            const int idx = tp.tid + kGemmThreads * p;
+            const int row = idx / (BN / 4), c4 = idx % (BN / 4);
+            rb[p] = load4<VEC_B>(b, k0 + row, n0 + 4 * c4, K, N);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int p = 0; p < Cfg::kA4; ++p) {
+            const int idx = tp.tid + kGemmThreads * p;
+            const int row = idx / (BM / 4), c4 = idx % (BM / 4);
+            *reinterpret_cast<float4*>(&lds_a[row * Cfg::kLdA + 4 * c4]) = ra[p];
+        }
+#pragma unroll
+        for (int p = 0; p < Cfg::kB4; ++p) {
+            const int idx = tp.tid + kGemmThreads * p;
+            const int row = idx / (BN / 4), c4 = idx % (BN / 4);
+            *reinterpret_cast<float4*>(&lds_b[row * Cfg::kLdB + 4 * c4]) = rb[p];
+        }
+    };
+
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += kBK) {
+        stage();
+        __syncthreads();
+        if (k0 + kBK < K) fetch(k0 + kBK);
+#pragma unroll
+        for (int kk = 0; kk < kBK / 2; ++kk) {
+            float fa[Cfg::kTilesM], fb[Cfg::kTilesN];
+            const int krow = 2 * kk + tp.half;
+#pragma unroll
+            for (int i = 0; i < Cfg::kTilesM; ++i) fa[i] = lds_a[krow * Cfg::kLdA + tp.wm0 + 32 * i + tp.l32];
+#pragma unroll
+            for (int j = 0; j < Cfg::kTilesN; ++j) fb[j] = lds_b[krow * Cfg::kLdB + tp.wn0 + 32 * j + tp.l32];
+#pragma unroll
+            for (int i = 0; i < Cfg::kTilesM; ++i)
+#pragma unroll
+                for (int j = 0; j < Cfg::kTilesN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace mcc
