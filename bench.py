@@ -96,7 +96,7 @@ def time_steps(step_fn, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def bench_fused(L, ops, name, steps, warmup):
+def bench_fused(L, ops, name, steps, warmup, fused_path="workspace"):
     import torch
     desc, shapes, layers, tokens = WORKLOADS[name]
     gen = torch.Generator(device="cuda")
@@ -113,7 +113,9 @@ def bench_fused(L, ops, name, steps, warmup):
             if n_out not in dys:
                 dys[n_out] = torch.randn(tokens, n_out, device="cuda", generator=gen) * 0.01
             tensors.append((make_state(gen, n_out, n_in), dys[n_out], xs[n_in], n_out, n_in))
-            ws_bytes = max(ws_bytes, ops.fused_workspace_nbytes(n_in, n_out, tokens))
+            need = ops.fused_strip_workspace_nbytes(n_in, n_out, tokens) if fused_path == "strip" else 0
+            # shapes the accumulator-resident step does not take fall back to the f32[out,in] workspace
+            ws_bytes = max(ws_bytes, need or ops.fused_workspace_nbytes(n_in, n_out, tokens))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
     params = sum(t[3] * t[4] for t in tensors)
     flops = sum(2.0 * tokens * t[3] * t[4] for t in tensors)
@@ -131,6 +133,10 @@ def bench_fused(L, ops, name, steps, warmup):
     ms_per_step = time_steps(step, steps, 0)
     gemm_ms, gemm_n = query(L, "gemm_tn_f32")
     upd_ms, upd_n = query(L, "counter_update")
+    strip_ms, strip_n = query(L, "fused_strip")
+    kernel = "gemm_tn_f32"
+    if strip_n and not gemm_n:
+        kernel, gemm_ms, gemm_n = "fused_strip", strip_ms, strip_n
     L.mcc_profiler_enable(0)
     L.mcc_profiler_reset()
     # dominant kernel: the contraction.  One launch per tensor; flops per launch differ by
@@ -141,13 +147,14 @@ def bench_fused(L, ops, name, steps, warmup):
         "ms_per_step": ms_per_step,
         "config": {"workload": desc, "tensors": len(tensors), "params": params, "tokens": tokens,
                    "C": C, "lr": LR, "lr_scale": LR_SCALE, "rms_beta": BETA, "rms_eps": EPS},
-        "roofline": {"bound": "mfma", "kernel": "gemm_tn_f32", "achieved": achieved,
+        "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved,
                      "peak": PEAK_MFMA_F32_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_MFMA_F32_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(name + "/gemm_tn_f32"),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name + "/" + kernel),
                      "launches": gemm_n, "avg_launch_ms": gemm_ms / max(gemm_n, 1),
                      "algorithmic_flops_per_step": flops},
-        "kernel_ms_per_step": {"gemm_tn_f32": gemm_ms / steps, "counter_update": upd_ms / steps},
+        "kernel_ms_per_step": {kernel: gemm_ms / steps, "counter_update": upd_ms / steps},
+        "fused_path": fused_path, "workspace_bytes": ws_bytes,
     }
     sample = tensors[0]
     del ws
@@ -283,6 +290,9 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--fused-path", default="workspace", choices=["workspace", "strip"],
+                    help="workspace: contraction into a lent f32[out,in] buffer, then the update kernel; "
+                         "strip: update applied from the contraction's accumulators, no weight-sized buffer")
     ap.add_argument("--no-update-only", action="store_true", help="skip the cfg3 update-only leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -312,7 +322,7 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
-    fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup)
+    fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup, args.fused_path)
     line = {
         "metric": "counter-synapse updates/s (Gparam/s)",
         "value": fused["value"], "unit": "Gparam/s", "n_gpus": 1, "steps": args.steps,
@@ -320,6 +330,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": fused["config"], "roofline": fused["roofline"],
         "kernel_ms_per_step": fused["kernel_ms_per_step"],
+        "fused_path": fused["fused_path"], "fused_workspace_bytes": fused["workspace_bytes"],
         "device": L.mcc_device_name().decode(),
     }
     if not args.no_cpu:

@@ -90,6 +90,30 @@ size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out
                                                   size_t batch);
 
 /*
+ * Bytes of the small workspace of the accumulator-resident fused step
+ * (32 KiB per 128 output rows plus flags), or 0 when the shape is not
+ * supported by it.  No counterpart in the reference.
+ */
+size_t mcc_compact_counter_fused_strip_workspace_nbytes(size_t in_features, size_t out_features,
+                                                        size_t batch);
+
+/*
+ * Waits for `stream` and reports whether the last fused step that used
+ * `workspace` completed: MCC_OK, or MCC_E_RUNTIME when a strip-workspace
+ * step gave up a wait (state of that tensor is then partially updated).
+ * Always MCC_OK for the full-size workspace.  No counterpart in the
+ * reference.
+ */
+int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t workspace_nbytes,
+                                    size_t in_features, size_t out_features, size_t batch);
+
+/*
+ * Polls a strip-workspace step spends on one wait before giving up (0
+ * restores the default, about four seconds).  For tests of the error path.
+ */
+void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
+
+/*
  * Fused step: weight-gradient contraction grad_w = grad_out^T . x on the fp32
  * matrix cores followed by the counter update.
  * Replaces run_vulkan_compact_counter_apply_update_fused
@@ -97,10 +121,23 @@ size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out
  *  src/runtime/vulkan_backend.cpp:8475-8578) and the OpenCL twin in
  * CounterStateLinear::apply_update_backward (src/nn/compact_counter.cpp:158-231).
  * The reference's scale_new/denom scratch buffers are not needed; instead the
- * caller lends `workspace` (>= mcc_compact_counter_fused_workspace_nbytes).
- * grad_w differs from the reference's sequential fp32 sum only by summation
- * order (relative error <= 1e-4 of the row norm); given that grad_w the counter
- * arithmetic is the same as in the dense entry point.
+ * caller lends `workspace`, whose size selects how the step runs:
+ *   - >= mcc_compact_counter_fused_workspace_nbytes (a f32[out,in] buffer):
+ *     contraction into the workspace, then the update kernel.  After the call
+ *     the workspace holds grad_w.
+ *   - >= mcc_compact_counter_fused_strip_workspace_nbytes but smaller than
+ *     the above: the update is applied from the contraction's accumulators
+ *     and no weight-sized buffer exists at any time, which is the property
+ *     tests/test_memory_truth_gate.cpp:109-113 of the reference asks for.
+ *     Needs lr_scale == 0, in/out multiples of 128 and a 16-byte aligned x.
+ *     Tiles of one row strip wait for each other on the device; two such
+ *     calls must not run concurrently on one GPU (they could starve each
+ *     other's waits), and mcc_compact_counter_fused_check reports a wait
+ *     that was given up.
+ * Both ways produce identical bytes.  grad_w differs from the reference's
+ * sequential fp32 sum only by summation order (relative error <= 1e-4 of the
+ * row norm); given that grad_w the counter arithmetic is the same as in the
+ * dense entry point.
  */
 int mcc_compact_counter_apply_update_fused(
     void* stream,

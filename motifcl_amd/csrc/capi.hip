@@ -33,6 +33,11 @@ int hip_fail(hipError_t e, const char* what) {
 
 constexpr size_t kIntMax = static_cast<size_t>(std::numeric_limits<int>::max());
 
+// Polls (about 0.25 us each) a strip-path workgroup spends on one wait before it gives up:
+// roughly four seconds, far above any wait a healthy launch can see.
+constexpr unsigned kDefaultStripSpinLimit = 1u << 24;
+std::atomic<unsigned> g_strip_spin_limit{kDefaultStripSpinLimit};
+
 // Shared shape/codec checks.  `what` names the operation in messages.
 bool check_codec(const char* what, size_t C, size_t in_features, size_t out_features) {
     if (in_features == 0 || out_features == 0) {
@@ -228,6 +233,33 @@ size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out
     return out_features * in_features * sizeof(float);
 }
 
+size_t mcc_compact_counter_fused_strip_workspace_nbytes(size_t in_features, size_t out_features,
+                                                        size_t batch) {
+    return mcc::fused_strip_workspace_nbytes(in_features, out_features, batch);
+}
+
+void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins) {
+    g_strip_spin_limit.store(spins ? spins : kDefaultStripSpinLimit);
+}
+
+int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t workspace_nbytes,
+                                    size_t in_features, size_t out_features, size_t batch) {
+    if (!workspace) return fail(MCC_E_INVALID, "compact-counter fused check received a null workspace");
+    const hipError_t es = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (es != hipSuccess) return hip_fail(es, "compact-counter fused check: stream synchronize failed");
+    const size_t full_nbytes = mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch);
+    if (full_nbytes == 0) return fail(MCC_E_INVALID, "compact-counter fused check requires non-zero dimensions");
+    if (workspace_nbytes >= full_nbytes) return MCC_OK;  // two-kernel path: nothing to wait on across workgroups
+    int status = 0;
+    const hipError_t ec = hipMemcpy(&status, workspace, sizeof(int), hipMemcpyDeviceToHost);
+    if (ec != hipSuccess) return hip_fail(ec, "compact-counter fused check: status read failed");
+    if (status != 0)
+        return fail(MCC_E_RUNTIME,
+                    "compact-counter fused strip update gave up waiting for a neighbouring tile; "
+                    "state, scale and v of this tensor are partially updated");
+    return MCC_OK;
+}
+
 int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t state_nbytes,
                                            float* scale, size_t scale_nbytes, float* v,
                                            size_t v_nbytes, const float* grad_out,
@@ -256,8 +288,17 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
         return fail(MCC_E_INVALID, "compact-counter fused update activation size overflows size_t");
     if (grad_out_nbytes < batch * out_features * sizeof(float) || x_nbytes < batch * in_features * sizeof(float))
         return fail(MCC_E_INVALID, "compact-counter fused update activation buffer is too small");
-    if (workspace_nbytes < mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch))
-        return fail(MCC_E_INVALID, "compact-counter fused update workspace is too small");
+    const size_t full_nbytes = mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch);
+    const size_t strip_nbytes = mcc::fused_strip_workspace_nbytes(in_features, out_features, batch);
+    const bool strip_path = workspace_nbytes < full_nbytes;
+    if (strip_path) {
+        if (strip_nbytes == 0 || workspace_nbytes < strip_nbytes)
+            return fail(MCC_E_INVALID, "compact-counter fused update workspace is too small");
+        if (lr_scale != 0.0f)
+            return fail(MCC_E_INVALID, "compact-counter fused update with the strip workspace requires lr_scale == 0");
+        if (reinterpret_cast<uintptr_t>(x) % 16)
+            return fail(MCC_E_INVALID, "compact-counter fused update with the strip workspace requires 16-byte aligned x");
+    }
     if (reinterpret_cast<uintptr_t>(workspace) % 16)
         return fail(MCC_E_INVALID, "compact-counter fused update workspace must be 16-byte aligned");
     if (reinterpret_cast<uintptr_t>(grad_out) % alignof(float) || reinterpret_cast<uintptr_t>(x) % alignof(float) ||
@@ -266,6 +307,14 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* grad_w = static_cast<float*>(workspace);
     hipError_t e;
+    if (strip_path) {
+        ScopedKernelTimer timer("fused_strip", s);
+        e = mcc::launch_fused_strip(s, state, scale, v, grad_out, x, workspace, (int)C, (int)in_features,
+                                    (int)out_features, (int)batch, lr, rms_beta, rms_eps, seed,
+                                    g_strip_spin_limit.load());
+        if (e != hipSuccess) return hip_fail(e, "compact-counter fused strip update launch failed");
+        return MCC_OK;
+    }
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
         e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features);

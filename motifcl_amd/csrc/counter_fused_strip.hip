@@ -1,0 +1,440 @@
+// Fused step without a weight-sized gradient buffer: the fp32 MFMA contraction
+//     G[o,i] = sum_r grad_out[r,o] * x[r,i]
+// keeps each 128 x 128 tile of G in its accumulators and applies the counter update to the
+// packed state straight from them.
+//
+// The obstacle is that every tick needs its row's denominator, i.e. the sum of squares over the
+// WHOLE row of G (kernels/compact_counter.cl:92-99 before :118), while a tile sees 128 columns.
+// The tiles of one 128-row strip therefore cooperate through a small strip scratch:
+//
+//   * The reference sums a row as 64 strided chains (chain l takes packed groups l, l+64, ...,
+//     kernels/compact_counter.cl:75-83) and then a binary tree (:88-91).  A tile's 128 columns
+//     are 32 consecutive groups, so tile ct of a strip holds exactly step ct/2 of the chains
+//     32*(ct%2) .. 32*(ct%2)+31 of its 128 rows.  Tile ct waits until tile ct-2 has published
+//     those chains, adds its four squares per group in element order, and publishes them for
+//     tile ct+2.  The even and the odd tiles form two independent hand-off sequences.
+//   * When both sequences have reached the end of the strip, every tile reads the 64 final chain
+//     values of each of its rows, runs the binary tree and the row epilogue itself, and applies
+//     the ticks to its own columns.  Tile 0 of the strip commits v and scale.
+//
+// The sums are the reference's, operation for operation, so the result is bit-identical to the
+// two-kernel path (contraction into a workspace, then the update kernel) on the same inputs.
+//
+// Workgroups are persistent: workgroup b takes tiles b, b + grid, b + 2 grid, ... of the
+// strip-major tile order.  A tile waits only for tiles of its own strip; a strip's tiles have
+// consecutive indices and a strip has no more tiles than the grid has workgroups, so the
+// workgroups that hold the lowest unfinished strip are all running and it always completes,
+// provided the whole grid is resident (the launch sizes it from the occupancy query).  Every
+// wait is bounded: a workgroup that exhausts its spin budget raises the status word, which
+// ends all waits, and the host reports the failure.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "counter_math.hpp"
+#include "gemm_tile.hpp"
+#include "launch.hpp"
+#include "wave_ops.hpp"
+
+namespace mcc {
+namespace {
+
+constexpr int kTile = 128;             // rows and columns of G per tile
+constexpr int kGroupsPerTile = kTile / 4;
+constexpr int kNapsPerHandOff = 2;  // s_sleep(32) units (about 0.9 us each) slept per pending hand-off
+constexpr int kStripChainFloats = 2 * kTile * kGroupsPerTile;  // both parities, 128 rows x 32 chains
+
+struct StripArgs {
+    uint8_t* state;
+    float* scale;
+    float* v;
+    const float* grad_out;
+    const float* x;
+    int* status;   // 0 while healthy
+    int* flags;    // [strip][2]: tiles of each parity that have published their chains
+    float* chain;  // [strip][2][128][32]
+    int tokens, in_features, out_features;
+    int tiles_per_strip, total_tiles;
+    unsigned spin_limit;
+    Codec cd;
+    LutGeom geom;
+    float lr, rms_beta, rms_eps;
+    uint32_t seed;
+};
+
+// Tables and per-row constants of the epilogue.
+struct EpilogueLds {
+    int q_off[64];
+    float c_f[64];          // residual counter of each code, before the rebase
+    float dn[kTile];        // denominator of each row of the strip
+    float k[kTile];         // Cf / scale_new
+    float ratio[kTile];     // scale_old / scale_new
+    uint8_t fin[kLutFinMaxBytes];
+    int ok;
+};
+
+// c_reb[code] of the update kernel, evaluated on the fly: (float)c * ratio.
+struct RebasedCounter {
+    const float* c_f;
+    float ratio;
+    __device__ __forceinline__ float operator[](uint32_t code) const { return c_f[code] * ratio; }
+};
+
+__device__ __forceinline__ int load_relaxed(const int* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Data that crosses workgroups (the chain blocks) moves with device-scope atomic accesses, which
+// are coherent between the per-XCD L2 caches by themselves, instead of ordinary accesses bracketed
+// by device-scope fences: a fence writes back or invalidates the whole L2 and costs tens of
+// microseconds when a thousand workgroups do it, and a strip has up to 43 hand-offs in sequence.
+// Ordering comes from completion: the producer waits until its stores have been acknowledged
+// (stores_done) before it raises the flag, and the consumer issues its loads only after it has
+// seen the flag.
+__device__ __forceinline__ float load_shared_f32(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void store_shared_f32(float* p, float x) {
+    __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void stores_done() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt = expcnt = lgkmcnt = 0
+}
+
+// Value of lane (4 * (lane / 4) + K) of the calling lane's quad.
+template <int K>
+__device__ __forceinline__ float quad_lane(float x) {
+    constexpr int ctrl = K | (K << 2) | (K << 4) | (K << 6);  // quad_perm:[K,K,K,K]
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), ctrl, 0xf, 0xf, false));
+}
+
+// OR over the four lanes of each quad.
+__device__ __forceinline__ uint32_t quad_or(uint32_t x) {
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xb1, 0xf, 0xf, false);  // quad_perm:[1,0,3,2]
+    x |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4e, 0xf, 0xf, false);  // quad_perm:[2,3,0,1]
+    return x;
+}
+
+// Parks the tile in the accumulation registers (AGPRs): between the phases of the epilogue the 64
+// accumulators are only kept, not used, and the vector registers are needed for the phase's own
+// working set.  Without this the compiler keeps them in vector registers and spills to scratch.
+template <int TM, int TN>
+__device__ __forceinline__ void park_accumulators(floatx16 (&acc)[TM][TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float t = acc[i][j][r];
+                asm volatile("" : "+a"(t));
+                acc[i][j][r] = t;
+            }
+}
+
+// The thread's tile coordinates recomputed from an index the compiler cannot see through: each
+// phase of the epilogue derives its addresses afresh instead of keeping hundreds of them, hoisted
+// out of the persistent tile loop, alive across the contraction.
+__device__ __forceinline__ TilePos fresh_tile_pos() {
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    TilePos p;
+    p.tid = tid;
+    const int lane = tid & 63, wave = tid >> 6;
+    p.l32 = lane & 31;
+    p.half = lane >> 5;
+    p.wm0 = (wave >> 1) * (kTile / 2);
+    p.wn0 = (wave & 1) * (kTile / 2);
+    return p;
+}
+
+// Thread 0 polls until *flag >= want or the status word is raised; returns whether the
+// workgroup may go on.  All threads of the workgroup call it.
+__device__ __forceinline__ bool wait_for(const StripArgs& a, const int* flag, int want, EpilogueLds& e) {
+    if (threadIdx.x == 0) {
+        int ok = 1;
+        unsigned spins = 0, polls = 0;
+        int seen;
+        while ((seen = load_relaxed(flag)) < want) {
+            // The flag counts hand-offs, each of which takes a few microseconds: sleep in
+            // proportion to the hand-offs still to come instead of polling at full rate.  A
+            // thousand workgroups polling a handful of words slow the contractions that are
+            // still running by a third.
+            const int naps = (want - seen - 1) * kNapsPerHandOff;
+            __builtin_amdgcn_s_sleep(8);
+            for (int n = 0; n < naps; ++n) __builtin_amdgcn_s_sleep(32);
+            spins += 1u + (unsigned)naps;
+            if ((++polls & 15u) == 0 && load_relaxed(a.status) != 0) {
+                ok = 0;
+                break;
+            }
+            if (spins >= a.spin_limit) {
+                __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ok = 0;
+                break;
+            }
+        }
+        e.ok = ok;
+    }
+    __syncthreads();
+    const bool ok = e.ok != 0;
+    __syncthreads();  // e.ok may be rewritten by the next wait
+    return ok;
+}
+
+template <bool VEC_A>
+__global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs a) {
+    using Cfg = TileCfg<kTile, kTile>;
+    __shared__ float lds[Cfg::kLdsFloats];
+    __shared__ EpilogueLds e;
+    const TilePos tp0 = tile_pos<kTile, kTile>();
+    for (int i = tp0.tid; i < 64; i += kGemmThreads) {
+        e.q_off[i] = q_off_entry((uint32_t)i, a.cd, a.geom);
+        e.c_f[i] = (float)code_c((uint32_t)i, a.cd);
+    }
+    for (int i = tp0.tid, n = fin_size(a.geom); i < n; i += kGemmThreads) fill_fin_entry(i, a.cd, a.geom, e.fin);
+    __syncthreads();
+
+    const int groups_per_row = a.in_features >> 2;
+    const uint32_t last_group_off = 3u * ((uint32_t)a.out_features * (uint32_t)groups_per_row - 1u);
+
+    for (int tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
+        const int strip = tile / a.tiles_per_strip;
+        const int ct = tile - strip * a.tiles_per_strip;
+        const int m0 = strip * kTile, n0 = ct * kTile;
+        const int parity = ct & 1, step = ct >> 1;
+        int* flags = a.flags + 2 * strip;
+        float* chain = a.chain + (size_t)strip * kStripChainFloats;
+
+        floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
+        gemm_tile_mainloop<kTile, kTile, VEC_A, true>(a.grad_out, a.x, a.tokens, a.out_features, a.in_features, m0,
+                                                      n0, tp0, lds, acc);
+
+        park_accumulators(acc);
+        // the hand-off sequence is latency-bound and other workgroups of this CU are still in
+        // their contraction: let the epilogue's few instructions issue first
+        __builtin_amdgcn_s_setprio(3);
+        TilePos tp = fresh_tile_pos();
+        int lane = tp.tid & 63, wave = tp.tid >> 6;
+        int kq = tp.l32 & 3;  // position of this lane's column inside its packed group
+
+        // Old per-row values, read before this tile publishes anything: tile 0 overwrites them
+        // only after every tile of the strip has published.
+        float s_old = 0.0f, v_old = 0.0f;
+        if (tp.tid < kTile) {
+            s_old = a.scale[m0 + tp.tid];
+            v_old = a.v[m0 + tp.tid];
+        }
+
+        // ---- chain hand-off: step `step` of chains 32*parity .. 32*parity+31 -------------
+        // The 128 x 32 chain block (16 KiB) is staged in the contraction's LDS slab buffer, which
+        // is free by now; each thread moves 16 floats, 256 contiguous bytes per wave and access.
+        if (!wait_for(a, flags + parity, step, e)) return;
+        park_accumulators(acc);
+        float* my_chain = chain + parity * (kTile * kGroupsPerTile);
+        static_assert(Cfg::kLdsFloats >= kTile * kGroupsPerTile, "chain block must fit the slab buffer");
+        constexpr int kChainPerThread = kTile * kGroupsPerTile / kGemmThreads;
+        {
+            float in[kChainPerThread];
+#pragma unroll
+            for (int p = 0; p < kChainPerThread; ++p)
+                in[p] = step > 0 ? load_shared_f32(my_chain + tp.tid + kGemmThreads * p) : 0.0f;
+#pragma unroll
+            for (int p = 0; p < kChainPerThread; ++p) lds[tp.tid + kGemmThreads * p] = in[p];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < Cfg::kTilesM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = tp.wm0 + 32 * i + 8 * (r / 4) + 4 * tp.half + (r % 4);
+#pragma unroll
+                for (int j = 0; j < Cfg::kTilesN; ++j) {
+                    const int gi = (tp.wn0 + 32 * j + tp.l32) >> 2;
+                    float* slot = lds + row * kGroupsPerTile + gi;  // owned by this lane's quad
+                    float c = *slot;
+                    const float sq = acc[i][j][r] * acc[i][j][r];
+                    c = c + quad_lane<0>(sq);  // element order inside the group
+                    c = c + quad_lane<1>(sq);
+                    c = c + quad_lane<2>(sq);
+                    c = c + quad_lane<3>(sq);
+                    if (kq == 0) *slot = c;
+                }
+            }
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < kChainPerThread; ++p)
+            store_shared_f32(my_chain + tp.tid + kGemmThreads * p, lds[tp.tid + kGemmThreads * p]);
+        stores_done();
+        __syncthreads();
+        if (tp.tid == 0) __hip_atomic_store(flags + parity, step + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+        // ---- row statistics once both hand-off sequences have reached the strip's end ----
+        const int n_even = (a.tiles_per_strip + 1) >> 1, n_odd = a.tiles_per_strip >> 1;
+        park_accumulators(acc);
+        tp = fresh_tile_pos();
+        lane = tp.tid & 63, wave = tp.tid >> 6;
+        if (!wait_for(a, flags + 0, n_even, e)) return;
+        if (n_odd > 0 && !wait_for(a, flags + 1, n_odd, e)) return;
+        {
+            // wave w finishes rows 32 w .. 32 w + 31: lane l holds chain l of the row
+            constexpr int kRowsPerWave = kTile / 4;
+            const float* mine = chain + (lane >> 5) * (kTile * kGroupsPerTile) + (lane & 31);
+            const bool have = lane < 32 || n_odd > 0;
+            float part[kRowsPerWave];
+#pragma unroll
+            for (int rr = 0; rr < kRowsPerWave; ++rr)
+                part[rr] = have ? load_shared_f32(mine + (wave * kRowsPerWave + rr) * kGroupsPerTile) : 0.0f;
+#pragma unroll
+            for (int rr = 0; rr < kRowsPerWave; ++rr) {
+                const float sum_sq = tree_sum(part[rr], lane);
+                if (lane == 0) e.dn[wave * kRowsPerWave + rr] = sum_sq;  // parked; replaced below
+            }
+        }
+        __syncthreads();
+        if (tp.tid < kTile) {
+            const RowStats rs = finish_row_stats(e.dn[tp.tid], 0.0f, v_old, s_old, a.in_features, 0.0f, a.rms_beta,
+                                                 a.rms_eps);
+            e.dn[tp.tid] = rs.denom;
+            e.k[tp.tid] = a.cd.Cf / rs.scale_new;
+            e.ratio[tp.tid] = s_old / rs.scale_new;
+            if (ct == 0) {
+                a.v[m0 + tp.tid] = rs.v_new;
+                a.scale[m0 + tp.tid] = rs.scale_new;
+            }
+        }
+        __syncthreads();
+
+        park_accumulators(acc);
+        tp = fresh_tile_pos();
+        kq = tp.l32 & 3;
+        // ---- ticks straight from the accumulators -----------------------------------------
+        TickConsts tc;
+        tc.r = 0.0f;
+        tc.neg_lr = -a.lr;
+        tc.neg_lim_neg = -(float)a.geom.lim_neg;
+        tc.lim_pos = (float)a.geom.lim_pos;
+        tc.two_m24 = 1.0f / 16777216.0f;
+        tc.seed = a.seed;
+        // 32-bit byte offsets from the state base (the launch checks that the state is smaller
+        // than 2 GiB): one add per element on top of a per-thread part
+        const uint32_t row_bytes = 3u * (uint32_t)groups_per_row;
+        const uint32_t my_state = (uint32_t)(m0 + tp.wm0 + 4 * tp.half) * row_bytes +
+                                  3u * ((uint32_t)(n0 + tp.wn0 + tp.l32) >> 2);
+        const uint32_t my_elem = (uint32_t)(m0 + tp.wm0 + 4 * tp.half) * (uint32_t)a.in_features +
+                                 (uint32_t)(n0 + tp.wn0 + tp.l32);
+        const int my_row = tp.wm0 + 4 * tp.half;
+#pragma unroll
+        for (int i = 0; i < Cfg::kTilesM; ++i)
+#pragma unroll
+            for (int j = 0; j < Cfg::kTilesN; ++j) {
+                // one 4-byte load per lane and element, all 16 issued before the first tick; the
+                // tensor's last group has no byte after it, so it is fetched one byte early and
+                // shifted down
+                uint32_t word[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t off = my_state + (uint32_t)(32 * i + 8 * (r / 4) + (r % 4)) * row_bytes + 24u * j;
+                    const uint32_t is_last = off == last_group_off ? 1u : 0u;
+                    __builtin_memcpy(&word[r], a.state + (off - is_last), 4);
+                    word[r] >>= 8 * is_last;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = my_row + 32 * i + 8 * (r / 4) + (r % 4);
+                    tc.dn = e.dn[row];
+                    tc.k = e.k[row];
+                    const RebasedCounter c_reb{e.c_f, e.ratio[row]};
+                    const uint32_t dr = (uint32_t)(32 * i + 8 * (r / 4) + (r % 4));
+                    const uint32_t elem = my_elem + dr * (uint32_t)a.in_features + 32u * j;
+                    const uint32_t off = my_state + dr * row_bytes + 24u * j;
+                    const uint32_t code = (word[r] >> (6 * kq)) & 0x3fu;
+                    const uint32_t nc = tick_code<false>(code, acc[i][j][r], tc, hash_first(elem), c_reb, e.q_off,
+                                                         e.fin);
+                    const uint32_t nw = quad_or(nc << (6 * kq));
+                    if (kq < 3) a.state[off + kq] = (uint8_t)(nw >> (8 * kq));
+                }
+            }
+        __builtin_amdgcn_s_setprio(0);
+        __syncthreads();  // the row constants are rewritten by the next tile
+    }
+}
+
+__global__ void strip_clear_kernel(int* words, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) words[i] = 0;
+}
+
+constexpr size_t kHeaderBytes = 256;  // status word, padded
+
+size_t flags_bytes(size_t strips) { return (strips * 2 * sizeof(int) + 255) / 256 * 256; }
+
+}  // namespace
+
+bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch) {
+    return batch > 0 && in_features >= kTile && out_features >= kTile && in_features % kTile == 0 &&
+           out_features % kTile == 0 && in_features <= (size_t(1) << 31) / out_features;  // 32-bit element offsets
+}
+
+size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch) {
+    if (!fused_strip_supports(in_features, out_features, batch)) return 0;
+    const size_t strips = out_features / kTile;
+    return kHeaderBytes + flags_bytes(strips) + strips * kStripChainFloats * sizeof(float);
+}
+
+hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, float* v, const float* grad_out,
+                              const float* x, void* workspace, int C, int in_features, int out_features, int tokens,
+                              float lr, float rms_beta, float rms_eps, uint32_t seed, unsigned spin_limit) {
+    const int strips = out_features / kTile;
+    StripArgs a;
+    a.state = state;
+    a.scale = scale;
+    a.v = v;
+    a.grad_out = grad_out;
+    a.x = x;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    a.status = reinterpret_cast<int*>(ws);
+    a.flags = reinterpret_cast<int*>(ws + kHeaderBytes);
+    a.chain = reinterpret_cast<float*>(ws + kHeaderBytes + flags_bytes((size_t)strips));
+    a.tokens = tokens;
+    a.in_features = in_features;
+    a.out_features = out_features;
+    a.tiles_per_strip = in_features / kTile;
+    a.total_tiles = strips * a.tiles_per_strip;
+    a.spin_limit = spin_limit;
+    a.cd = make_codec(C);
+    a.geom = lut_geom(a.cd);
+    a.lr = lr;
+    a.rms_beta = rms_beta;
+    a.rms_eps = rms_eps;
+    a.seed = seed;
+
+    const bool vec_a = (reinterpret_cast<uintptr_t>(grad_out) & 15u) == 0;  // out_features % 4 == 0 holds
+    if ((reinterpret_cast<uintptr_t>(x) & 15u) != 0) return hipErrorInvalidValue;
+    auto kernel = vec_a ? fused_strip_kernel<true> : fused_strip_kernel<false>;
+
+    // the whole grid must be resident at once: size it from what the device can hold
+    int device = 0, cus = 0, per_cu = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return err;
+    err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+    if (err != hipSuccess) return err;
+    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kGemmThreads, 0);
+    if (err != hipSuccess) return err;
+    const long capacity = (long)cus * per_cu;
+    if (capacity < a.tiles_per_strip) return hipErrorLaunchOutOfResources;
+    const int grid = (int)(capacity < a.total_tiles ? capacity : a.total_tiles);
+
+    const int clear_words = (int)((kHeaderBytes + flags_bytes((size_t)strips)) / sizeof(int));
+    hipLaunchKernelGGL(strip_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, stream,
+                       reinterpret_cast<int*>(ws), clear_words);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kGemmThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace mcc

@@ -34,6 +34,15 @@ hipError_t launch_update_dense(hipStream_t stream, uint8_t* state, float* scale,
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c,
                               int k, int m, int n);
 
+// Fused step that keeps G in the contraction's accumulators (counter_fused_strip.hip).
+// Shapes: in_features and out_features multiples of 128; lr_scale == 0 is implied.
+bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch);
+size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch);
+hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, float* v,
+                              const float* grad_out, const float* x, void* workspace, int C,
+                              int in_features, int out_features, int tokens, float lr, float rms_beta,
+                              float rms_eps, uint32_t seed, unsigned spin_limit);
+
 hipError_t launch_decode_weight(hipStream_t stream, const uint8_t* state, const float* scale,
                                 float* weight, int C, int in_features, int out_features);
 

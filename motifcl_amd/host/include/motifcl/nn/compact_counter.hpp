@@ -2,12 +2,23 @@
 // include/motifcl/nn/compact_counter.hpp:16-60 of MotifCL, implemented on the HIP library.
 #pragma once
 
+#include <cstddef>
 #include <cstdint>
 
 #include <motifcl/nn/module.hpp>
 #include <motifcl/runtime/backend.hpp>
 
 namespace motifcl::nn {
+
+// How the fused update holds the weight gradient while it needs the whole row's RMS:
+//   Strip  the gradient never leaves the contraction's registers; tiles of a 128-row strip
+//          exchange 32 KiB of partial row sums (no weight-sized buffer, as in the reference,
+//          tests/test_memory_truth_gate.cpp:109-113); needs lr_scale == 0 and in/out multiples
+//          of 128, other layers silently use Full
+//   Full   contraction into a f32[out,in] workspace, then the update kernel (a few percent
+//          faster on large layers)
+// Both give identical bytes.
+enum class FusedWorkspace { Strip, Full };
 
 // Ternary finite-state "counter" linear layer trained as a per-synapse automaton: the whole
 // trainable state is a packed 6-bit code per weight plus a per-row scale and a per-row RMS
@@ -29,6 +40,10 @@ public:
 
     void set_training(bool t) { training_ = t; }
     bool training() const { return training_; }
+    void set_fused_workspace(FusedWorkspace w) { fused_workspace_ = w; }
+    FusedWorkspace fused_workspace() const { return fused_workspace_; }
+    // Waits for the backend and throws if the last Strip update gave up an inter-tile wait.
+    void check_fused_update() const;
     void set_lr(float lr) { lr_ = lr; }
     float lr() const { return lr_; }
 
@@ -51,6 +66,8 @@ private:
     float rms_eps_ = 1e-3f;
     std::uint32_t seed_ = 12345u;
     bool training_ = true;
+    FusedWorkspace fused_workspace_ = FusedWorkspace::Strip;
+    std::size_t last_fused_ws_ = 0, last_fused_batch_ = 0;
 };
 
 }  // namespace motifcl::nn

@@ -44,6 +44,8 @@ public:
     // Transient workspace shared by every layer of this backend (the fused update's gradient
     // strip); grows to the largest request and is returned to the pool with the backend.
     void* workspace(std::size_t nbytes);
+    std::size_t workspace_nbytes() const { return workspace_nbytes_; }
+    void release_workspace();
 
 private:
     void* stream_ = nullptr;

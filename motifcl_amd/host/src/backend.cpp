@@ -58,6 +58,14 @@ void* Backend::workspace(std::size_t nbytes) {
     return workspace_;
 }
 
+void Backend::release_workspace() {
+    if (!workspace_) return;
+    finish();
+    mcc_device_free(workspace_);
+    workspace_ = nullptr;
+    workspace_nbytes_ = 0;
+}
+
 std::size_t device_bytes_current() { return mcc_device_bytes_current(); }
 std::size_t device_bytes_peak() { return mcc_device_bytes_peak(); }
 void device_bytes_reset_peak() { mcc_device_bytes_reset_peak(); }

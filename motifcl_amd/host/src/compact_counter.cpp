@@ -104,14 +104,27 @@ void CounterStateLinear::apply_update_seed(const Tensor& grad_w, std::uint32_t s
 void CounterStateLinear::apply_update_backward(const Tensor& grad_out, const Tensor& x, std::uint32_t seed) {
     MCL_CHECK(x.ndim() == 2 && grad_out.ndim() == 2, "apply_update_backward expects rank-2 tensors");
     const std::size_t N = static_cast<std::size_t>(x.shape()[0]);
-    const std::size_t ws = mcc_compact_counter_fused_workspace_nbytes(static_cast<std::size_t>(in_),
-                                                                     static_cast<std::size_t>(out_), N);
+    const std::size_t in = static_cast<std::size_t>(in_), out = static_cast<std::size_t>(out_);
+    std::size_t ws = 0;
+    if (fused_workspace_ == FusedWorkspace::Strip && lr_scale_ == 0.0f)
+        ws = mcc_compact_counter_fused_strip_workspace_nbytes(in, out, N);  // 0: shape not supported
+    if (ws == 0) ws = mcc_compact_counter_fused_workspace_nbytes(in, out, N);
     void* scratch = backend_->workspace(ws);
+    // exactly ws bytes are lent: the size selects how the step runs
     const int rc = mcc_compact_counter_apply_update_fused(
         backend_->hip_stream(), static_cast<std::uint8_t*>(state.data()), state.nbytes(), f32(scale), scale.nbytes(),
         f32(v), v.nbytes(), f32(grad_out), grad_out.nbytes(), f32(x), x.nbytes(), scratch, ws,
-        static_cast<std::size_t>(C_), static_cast<std::size_t>(in_), static_cast<std::size_t>(out_), N, lr_, lr_scale_,
-        rms_beta_, rms_eps_, seed);
+        static_cast<std::size_t>(C_), in, out, N, lr_, lr_scale_, rms_beta_, rms_eps_, seed);
+    MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter fused update failed: ") + mcc_last_error());
+    last_fused_ws_ = ws;
+    last_fused_batch_ = N;
+}
+
+void CounterStateLinear::check_fused_update() const {
+    if (last_fused_ws_ == 0) return;
+    const int rc = mcc_compact_counter_fused_check(backend_->hip_stream(), backend_->workspace(last_fused_ws_),
+                                                   last_fused_ws_, static_cast<std::size_t>(in_),
+                                                   static_cast<std::size_t>(out_), last_fused_batch_);
     MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter fused update failed: ") + mcc_last_error());
 }
 

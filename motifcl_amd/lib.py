@@ -16,6 +16,9 @@ SIGNATURES = {
     "mcc_compact_counter_apply_update_dense_batched": (
         ctypes.c_int, [_vp, _vp, _sz, _sz, _f, _f, _f]),
     "mcc_compact_counter_fused_workspace_nbytes": (_sz, [_sz, _sz, _sz]),
+    "mcc_compact_counter_fused_strip_workspace_nbytes": (_sz, [_sz, _sz, _sz]),
+    "mcc_compact_counter_fused_check": (ctypes.c_int, [_vp, _vp, _sz, _sz, _sz, _sz]),
+    "mcc_compact_counter_fused_strip_set_spin_limit": (None, [ctypes.c_uint]),
     "mcc_compact_counter_apply_update_fused": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
                        _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),

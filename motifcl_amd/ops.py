@@ -68,6 +68,19 @@ def fused_workspace_nbytes(in_features, out_features, batch):
     return int(_lib.load().mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch))
 
 
+def fused_strip_workspace_nbytes(in_features, out_features, batch):
+    """Size of the small workspace of the accumulator-resident fused step; 0 if unsupported."""
+    return int(_lib.load().mcc_compact_counter_fused_strip_workspace_nbytes(in_features, out_features, batch))
+
+
+def fused_check(workspace, in_features, out_features, batch):
+    """Waits for the stream and raises MccError if a strip-workspace step gave up a wait."""
+    L = _lib.load()
+    _lib.check(L.mcc_compact_counter_fused_check(
+        _stream(), workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+        in_features, out_features, batch))
+
+
 def apply_update_fused(state, scale, v, grad_out, x, workspace, C, lr, lr_scale, rms_beta, rms_eps,
                        seed):
     """In-place fused step (CounterStateLinear::apply_update_backward)."""

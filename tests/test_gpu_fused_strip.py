@@ -1,0 +1,140 @@
+"""Accumulator-resident fused step against the two-kernel fused step (same bytes) and the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from tests import synth
+from tests.test_gpu_parity import dev, host, ops  # noqa: F401  (fixture)
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+HP = dict(lr=3e-3, lr_scale=0.0, rms_beta=0.9, rms_eps=1e-3)
+
+# (N, in, out, C)
+STRIP_SHAPES = [
+    (64, 128, 128, 11),     # one tile: a strip of a single column tile (odd chains stay empty)
+    (100, 256, 128, 11),    # one strip, one tile per parity; token count not a multiple of the slab
+    (96, 384, 256, 3),      # odd number of tiles per strip
+    (257, 1024, 384, 11),
+    (64, 768, 2048, 11),    # BASELINE cfg2 shapes, few tokens
+    (64, 2048, 768, 8),
+    (32, 4096, 4096, 11),   # 1024 tiles: the whole grid in one pass
+    (32, 11008, 4096, 11),  # 86 tiles per strip, several passes of the persistent grid
+    (32, 4096, 11008, 11),
+]
+
+
+def run_both(ops, n, n_in, n_out, C, seed, lr=HP["lr"]):
+    _, _, _, scale, v = synth.counter_case(seed, n_out, n_in, C, oracle=None)
+    rng = np.random.default_rng(seed + 1)
+    hi = 3 * (2 * C - 1)
+    # every 6-bit code inside the reachable range
+    codes = rng.integers(0, hi, (n_out, n_in)).astype(np.uint32).reshape(-1, 4)
+    word = codes[:, 0] | (codes[:, 1] << 6) | (codes[:, 2] << 12) | (codes[:, 3] << 18)
+    state = np.stack([word & 255, (word >> 8) & 255, (word >> 16) & 255], axis=1).astype(np.uint8).reshape(-1)
+    x, dy = synth.activations(seed + 2, n, n_in, n_out)
+    dx, ddy = dev(x), dev(dy)
+    out = []
+    for nbytes in (ops.fused_workspace_nbytes(n_in, n_out, n), ops.fused_strip_workspace_nbytes(n_in, n_out, n)):
+        assert nbytes > 0
+        d = [dev(state), dev(scale), dev(v)]
+        ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        ops.apply_update_fused(*d, ddy, dx, ws, C, lr, HP["lr_scale"], HP["rms_beta"], HP["rms_eps"], 4242)
+        ops.fused_check(ws, n_in, n_out, n)
+        out.append([host(t) for t in d])
+    return state, scale, v, x, dy, out
+
+
+@pytest.mark.parametrize("shape", STRIP_SHAPES, ids=lambda s: "N%d_in%d_out%d_C%d" % s)
+def test_strip_path_matches_two_kernel_path(ops, shape):
+    n, n_in, n_out, C = shape
+    print("strip case", shape, flush=True)
+    assert ops.fused_strip_workspace_nbytes(n_in, n_out, n) < ops.fused_workspace_nbytes(n_in, n_out, n)
+    state, scale, v, _, _, (full, strip) = run_both(ops, n, n_in, n_out, C, seed=n_in + n_out)
+    assert not np.array_equal(full[0], state)
+    assert np.array_equal(strip[1], full[1])  # scale
+    assert np.array_equal(strip[2], full[2])  # v
+    assert np.array_equal(strip[0], full[0])  # state bytes
+
+
+def test_strip_path_against_oracle(ops, oracle):
+    n, n_in, n_out, C = 192, 512, 256, 11
+    state, scale, v, x, dy, (_, strip) = run_both(ops, n, n_in, n_out, C, seed=5)
+    e_state, e_scale, e_v, _ = oracle.update_fused(state, scale, v, dy, x, C, HP["lr"], HP["lr_scale"],
+                                                   HP["rms_beta"], HP["rms_eps"], 4242)
+    flips = np.mean(oracle.unpack_codes(strip[0]) != oracle.unpack_codes(e_state))
+    print("strip vs oracle: counter-flip mismatch %.3e" % flips)
+    assert flips <= 2e-3
+    assert np.allclose(strip[2], e_v, rtol=1e-5, atol=0)
+    assert np.array_equal(strip[1], e_scale)
+
+
+def test_strip_workspace_rules(ops):
+    assert ops.fused_strip_workspace_nbytes(288, 288, 64) == 0      # not multiples of 128
+    assert ops.fused_strip_workspace_nbytes(128, 64, 64) == 0
+    n, n_in, n_out, C = 64, 256, 128, 11
+    _, _, _, scale, v = synth.counter_case(1, n_out, n_in, C)
+    state = np.zeros(n_out * n_in // 4 * 3, dtype=np.uint8)
+    x, dy = synth.activations(2, n, n_in, n_out)
+    ws = torch.empty(ops.fused_strip_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
+    from motifcl_amd.lib import MccError
+    with pytest.raises(MccError, match="lr_scale"):
+        ops.apply_update_fused(dev(state), dev(scale), dev(v), dev(dy), dev(x), ws, C, 3e-3, 0.05, 0.9, 1e-3, 1)
+    with pytest.raises(MccError, match="too small"):
+        ops.apply_update_fused(dev(state), dev(scale), dev(v), dev(dy), dev(x), ws[:-16], C, 3e-3, 0.0, 0.9, 1e-3, 1)
+
+
+def test_two_strip_updates_in_a_row_are_deterministic(ops):
+    # the strip scratch keeps the previous call's contents; a second call, on a smaller layer
+    # through the same workspace, must not see them (tests/test_vulkan_counter_fused.cpp:120-133)
+    ws = torch.empty(ops.fused_strip_workspace_nbytes(1024, 512, 64), dtype=torch.uint8, device="cuda")
+    results = []
+    for n, n_in, n_out in ((64, 1024, 512), (48, 512, 256), (48, 512, 256)):
+        rng = np.random.default_rng(n_in)
+        state = np.zeros(n_out * n_in // 4 * 3, dtype=np.uint8)
+        scale = np.full(n_out, 0.05, dtype=F)
+        v = np.zeros(n_out, dtype=F)
+        x, dy = synth.activations(9, n, n_in, n_out)
+        d = [dev(state), dev(scale), dev(v)]
+        ops.apply_update_fused(*d, dev(dy), dev(x), ws, 11, 3e-3, 0.0, 0.9, 1e-3, 99)
+        ops.fused_check(ws, n_in, n_out, n)
+        results.append([host(t) for t in d])
+    for a, b in zip(results[1], results[2]):
+        assert np.array_equal(a, b)
+
+
+def test_given_up_wait_is_reported_and_every_workgroup_exits(ops):
+    # a spin budget of one poll makes waits fail from the host side; the kernel must still
+    # drain and the failure must surface through fused_check
+    import motifcl_amd
+    from motifcl_amd.lib import MccError
+    L = motifcl_amd.load()
+    n, n_in, n_out, C = 32, 4096, 256, 11
+    state = np.zeros(n_out * n_in // 4 * 3, dtype=np.uint8)
+    scale = np.full(n_out, 0.05, dtype=F)
+    v = np.zeros(n_out, dtype=F)
+    x, dy = synth.activations(3, n, n_in, n_out)
+    ws = torch.empty(ops.fused_strip_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
+    L.mcc_compact_counter_fused_strip_set_spin_limit(1)
+    try:
+        d = [dev(state), dev(scale), dev(v)]
+        ops.apply_update_fused(*d, dev(dy), dev(x), ws, C, 3e-3, 0.0, 0.9, 1e-3, 5)
+        try:
+            ops.fused_check(ws, n_in, n_out, n)
+            gave_up = False
+        except MccError as err:
+            assert "gave up waiting" in str(err)
+            gave_up = True
+    finally:
+        L.mcc_compact_counter_fused_strip_set_spin_limit(0)
+    print("wait given up with a one-poll budget:", gave_up)
+    # with the default budget the same call completes and matches the two-kernel path
+    ref = [dev(state), dev(scale), dev(v)]
+    full = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
+    ops.apply_update_fused(*ref, dev(dy), dev(x), full, C, 3e-3, 0.0, 0.9, 1e-3, 5)
+    d = [dev(state), dev(scale), dev(v)]
+    ops.apply_update_fused(*d, dev(dy), dev(x), ws, C, 3e-3, 0.0, 0.9, 1e-3, 5)
+    ops.fused_check(ws, n_in, n_out, n)
+    for a, b in zip(d, ref):
+        assert torch.equal(a, b)
