@@ -161,6 +161,47 @@ def bench_fused(L, ops, name, steps, warmup, fused_path="workspace"):
     return out, sample, tokens
 
 
+def bench_layer_products(L, ops, name, steps, warmup):
+    """The other two contractions of a counter layer step (forward, input gradient) on the workload's shapes."""
+    import torch
+    desc, shapes, layers, tokens = WORKLOADS[name]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(2)
+    out = {}
+    xs, dys = {}, {}
+    tensors = []
+    for (n_out, n_in) in shapes:  # one layer's shapes: the products keep no state between calls
+        if n_in not in xs:
+            xs[n_in] = torch.randn(tokens, n_in, device="cuda", generator=gen)
+        if n_out not in dys:
+            dys[n_out] = torch.randn(tokens, n_out, device="cuda", generator=gen) * 0.01
+        tensors.append((make_state(gen, n_out, n_in), n_out, n_in))
+    flops = sum(2.0 * tokens * t[1] * t[2] for t in tensors)
+    y = {n: torch.empty(tokens, n, device="cuda") for n in set(t[1] for t in tensors) | set(t[2] for t in tensors)}
+
+    def step(_):
+        for (state, scale, v), n_out, n_in in tensors:
+            ops.forward(xs[n_in], state, scale, C, n_out, out=y[n_out])
+            ops.backward_input(dys[n_out], state, scale, C, n_in, out=y[n_in])
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    L.mcc_profiler_reset()
+    L.mcc_profiler_enable(1)
+    time_steps(step, steps, 0)
+    for kernel in ("counter_forward", "counter_backward_input"):
+        ms, n = query(L, kernel)
+        tf = flops * steps / (ms * 1e-3) / 1e12
+        out[kernel] = {"ms_per_step": ms / steps, "launches": n, "achieved": tf, "unit": "TFLOP/s",
+                       "frac": tf / PEAK_MFMA_F32_TFLOPS}
+    L.mcc_profiler_enable(0)
+    L.mcc_profiler_reset()
+    out["tensors"] = len(tensors)
+    out["tokens"] = tokens
+    return out
+
+
 def bench_update_only(L, ops, steps, warmup):
     import torch
     shapes = layer_shapes(4096, 11008)
@@ -337,6 +378,8 @@ def main():
         line["cpu_baseline"] = cpu_baseline_fused(fused_sample, tokens, args.cpu_rows)
         line["parity"] = parity_leg(ops)
     del fused_sample
+    torch.cuda.empty_cache()
+    line["layer_products"] = bench_layer_products(L, ops, args.workload, max(2, args.steps // 2), 1)
     torch.cuda.empty_cache()
     if not args.no_update_only:
         uo, uo_sample = bench_update_only(L, ops, args.steps, args.warmup)

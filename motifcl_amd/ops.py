@@ -119,20 +119,20 @@ def decode_weight(state, scale, C, in_features, out_features):
     return w
 
 
-def forward(x, state, scale, C, out_features):
+def forward(x, state, scale, C, out_features, out=None):
     L = _lib.load()
     batch, in_features = x.shape
-    y = torch.empty((batch, out_features), dtype=torch.float32, device=x.device)
+    y = out if out is not None else torch.empty((batch, out_features), dtype=torch.float32, device=x.device)
     _lib.check(L.mcc_compact_counter_forward_u8(
         _stream(), *_buf(x, torch.float32), *_buf(state, torch.uint8), *_buf(scale, torch.float32),
         *_buf(y, torch.float32), batch, in_features, out_features, C))
     return y
 
 
-def backward_input(grad_out, state, scale, C, in_features):
+def backward_input(grad_out, state, scale, C, in_features, out=None):
     L = _lib.load()
     batch, out_features = grad_out.shape
-    gx = torch.empty((batch, in_features), dtype=torch.float32, device=grad_out.device)
+    gx = out if out is not None else torch.empty((batch, in_features), dtype=torch.float32, device=grad_out.device)
     _lib.check(L.mcc_compact_counter_backward_input_u8(
         _stream(), *_buf(state, torch.uint8), *_buf(scale, torch.float32),
         *_buf(grad_out, torch.float32), *_buf(gx, torch.float32),
