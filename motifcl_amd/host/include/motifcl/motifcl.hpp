@@ -7,4 +7,5 @@
 #include <motifcl/nn/compact_counter.hpp>
 #include <motifcl/ops/matmul.hpp>
 #include <motifcl/runtime/backend.hpp>
+#include <motifcl/serialization.hpp>
 #include <motifcl/tensor/tensor.hpp>

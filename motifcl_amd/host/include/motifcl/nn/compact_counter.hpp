@@ -37,6 +37,9 @@ public:
     void apply_update_backward(const Tensor& grad_out, const Tensor& x, std::uint32_t seed);  // fused
     Tensor backward_input_from_state(const Tensor& grad_out) const;   // grad_x [N, in]
     std::uint32_t next_seed() { return seed_++; }
+    // Resume rule of tools/train_ternary15m.cpp:112-121: seeds advance once per update, so a
+    // layer built with seed `base` continues an interrupted run from `base + completed_steps`.
+    void set_next_seed(std::uint32_t seed) { seed_ = seed; }
 
     void set_training(bool t) { training_ = t; }
     bool training() const { return training_; }
