@@ -203,6 +203,33 @@ def bench_layer_products(L, ops, name, steps, warmup):
     return out
 
 
+def bench_side_optimizer(L, ops, steps, warmup):
+    """Adam on one large FP32 tensor: 16 B read + 12 B written per element."""
+    import torch
+    n = 1 << 28  # 1 GiB per buffer
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    p = torch.randn(n, device="cuda", generator=gen)
+    g = torch.randn(n, device="cuda", generator=gen) * 0.01
+    m = torch.zeros(n, device="cuda")
+    v = torch.zeros(n, device="cuda")
+    for i in range(warmup):
+        ops.adam_update(p, g, m, v, 3e-4, 0.9, 0.95, 1e-8, i + 1, 0.01)
+    torch.cuda.synchronize()
+    L.mcc_profiler_reset()
+    L.mcc_profiler_enable(1)
+    time_steps(lambda i: ops.adam_update(p, g, m, v, 3e-4, 0.9, 0.95, 1e-8, warmup + i + 1, 0.01), steps, 0)
+    ms, launches = query(L, "adam_update")
+    L.mcc_profiler_enable(0)
+    L.mcc_profiler_reset()
+    achieved = 28.0 * n * launches / (ms * 1e-3) / 1e9
+    return {"workload": "adam_update_fast on one f32 tensor of 2^28 elements", "ms_per_launch": ms / launches,
+            "value": n * launches / (ms * 1e-3) / 1e9, "unit": "Gparam/s",
+            "roofline": {"bound": "hbm", "kernel": "adam_kernel", "achieved": achieved, "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None,
+                         "algorithmic_bytes_per_param": 28.0}}
+
+
 def bench_update_only(L, ops, steps, warmup):
     import torch
     shapes = layer_shapes(4096, 11008)
@@ -379,6 +406,8 @@ def main():
         line["cpu_baseline"] = cpu_baseline_fused(fused_sample, tokens, args.cpu_rows)
         line["parity"] = parity_leg(ops)
     del fused_sample
+    torch.cuda.empty_cache()
+    line["side_optimizer"] = bench_side_optimizer(L, ops, max(3, args.steps), 2)
     torch.cuda.empty_cache()
     line["layer_products"] = bench_layer_products(L, ops, args.workload, max(2, args.steps // 2), 1)
     torch.cuda.empty_cache()

@@ -206,6 +206,21 @@ int mcc_compact_counter_backward_input_u8(
     size_t batch, size_t in_features, size_t out_features, size_t C);
 
 /*
+ * FP32 side optimizers for the non-counter tensors of a counter model
+ * (embedding, norm gains).  Replace sgd_update and adam_update_fast
+ * (include/motifcl/ops/optim.hpp, src/ops/optim.cpp:17-86; kernels
+ * kernels/optim.cl:1-7,31-53).  `n` counts elements; all buffers hold n floats.
+ * Adam: step >= 1; the bias corrections 1/(1 - beta^step) are computed on the
+ * host in binary32 as the reference does (src/ops/optim.cpp:70-71).
+ */
+int mcc_sgd_update_f32(void* stream, float* param, size_t param_nbytes, const float* grad,
+                       size_t grad_nbytes, size_t n, float lr);
+int mcc_adam_update_f32(void* stream, float* param, size_t param_nbytes, const float* grad,
+                        size_t grad_nbytes, float* m, size_t m_nbytes, float* v, size_t v_nbytes,
+                        size_t n, float lr, float beta1, float beta2, float eps, int step,
+                        float weight_decay);
+
+/*
  * Device-resident storage.  Replaces the pooled VulkanRuntime::create_buffer /
  * Storage allocator (src/runtime/vulkan_backend.cpp:4663-4719,6462-6510;
  * src/tensor/storage.cpp:35-79): freed blocks are kept in power-of-two buckets

@@ -521,6 +521,43 @@ int mcc_memcpy_d2h(void* stream, void* dst, const void* src, size_t nbytes) {
     return MCC_OK;
 }
 
+int mcc_sgd_update_f32(void* stream, float* param, size_t param_nbytes, const float* grad, size_t grad_nbytes,
+                       size_t n, float lr) {
+    if (n == 0) return fail(MCC_E_INVALID, "sgd_update requires a non-empty tensor");
+    if (!param || !grad) return fail(MCC_E_INVALID, "sgd_update received a null buffer");
+    if (n > std::numeric_limits<size_t>::max() / sizeof(float) || param_nbytes < n * sizeof(float) ||
+        grad_nbytes < n * sizeof(float))
+        return fail(MCC_E_INVALID, "sgd_update shape mismatch: a buffer is smaller than n floats");
+    if (reinterpret_cast<uintptr_t>(param) % alignof(float) || reinterpret_cast<uintptr_t>(grad) % alignof(float))
+        return fail(MCC_E_INVALID, "sgd_update buffers must be 4-byte aligned");
+    ScopedKernelTimer timer("sgd_update", static_cast<hipStream_t>(stream));
+    const hipError_t e = mcc::launch_sgd_update(static_cast<hipStream_t>(stream), param, grad, n, lr);
+    if (e != hipSuccess) return hip_fail(e, "sgd_update launch failed");
+    return MCC_OK;
+}
+
+int mcc_adam_update_f32(void* stream, float* param, size_t param_nbytes, const float* grad, size_t grad_nbytes,
+                        float* m, size_t m_nbytes, float* v, size_t v_nbytes, size_t n, float lr, float beta1,
+                        float beta2, float eps, int step, float weight_decay) {
+    if (n == 0) return fail(MCC_E_INVALID, "adam_update requires a non-empty tensor");
+    if (step <= 0) return fail(MCC_E_INVALID, "adam_update step must be positive");
+    if (!param || !grad || !m || !v) return fail(MCC_E_INVALID, "adam_update received a null buffer");
+    if (n > std::numeric_limits<size_t>::max() / sizeof(float)) return fail(MCC_E_INVALID, "adam_update size overflows");
+    const size_t need = n * sizeof(float);
+    if (param_nbytes < need || grad_nbytes < need || m_nbytes < need || v_nbytes < need)
+        return fail(MCC_E_INVALID, "adam_update shape mismatch: a buffer is smaller than n floats");
+    if (reinterpret_cast<uintptr_t>(param) % alignof(float) || reinterpret_cast<uintptr_t>(grad) % alignof(float) ||
+        reinterpret_cast<uintptr_t>(m) % alignof(float) || reinterpret_cast<uintptr_t>(v) % alignof(float))
+        return fail(MCC_E_INVALID, "adam_update buffers must be 4-byte aligned");
+    const float inv_bias1 = 1.0f / (1.0f - std::pow(beta1, static_cast<float>(step)));
+    const float inv_bias2 = 1.0f / (1.0f - std::pow(beta2, static_cast<float>(step)));
+    ScopedKernelTimer timer("adam_update", static_cast<hipStream_t>(stream));
+    const hipError_t e = mcc::launch_adam_update(static_cast<hipStream_t>(stream), param, grad, m, v, n, lr, beta1,
+                                                 beta2, eps, inv_bias1, inv_bias2, weight_decay);
+    if (e != hipSuccess) return hip_fail(e, "adam_update launch failed");
+    return MCC_OK;
+}
+
 int mcc_memset_zero(void* stream, void* dst, size_t nbytes) {
     if (nbytes == 0) return MCC_OK;
     if (!dst) return fail(MCC_E_INVALID, "memset received a null pointer");

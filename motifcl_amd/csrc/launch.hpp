@@ -56,4 +56,10 @@ hipError_t launch_backward_input(hipStream_t stream, const float* grad_out, cons
                                  const float* scale, float* grad_x, int C, int batch,
                                  int in_features, int out_features);
 
+// param -= lr * grad; Adam with precomputed bias corrections (side_optim.hip)
+hipError_t launch_sgd_update(hipStream_t stream, float* param, const float* grad, size_t n, float lr);
+hipError_t launch_adam_update(hipStream_t stream, float* param, const float* grad, float* m, float* v,
+                              size_t n, float lr, float beta1, float beta2, float eps, float inv_bias1,
+                              float inv_bias2, float weight_decay);
+
 }  // namespace mcc

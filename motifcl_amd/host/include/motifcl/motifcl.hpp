@@ -6,6 +6,7 @@
 #include <motifcl/core/shape.hpp>
 #include <motifcl/nn/compact_counter.hpp>
 #include <motifcl/ops/matmul.hpp>
+#include <motifcl/ops/optim.hpp>
 #include <motifcl/runtime/backend.hpp>
 #include <motifcl/serialization.hpp>
 #include <motifcl/tensor/tensor.hpp>

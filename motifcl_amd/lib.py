@@ -28,6 +28,9 @@ SIGNATURES = {
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _sz]),
     "mcc_compact_counter_backward_input_u8": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _sz]),
+    "mcc_sgd_update_f32": (ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _f]),
+    "mcc_adam_update_f32": (ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _f, _f, _f, _f,
+                                           ctypes.c_int, _f]),
     "mcc_device_alloc": (ctypes.c_int, [ctypes.POINTER(_vp), _sz]),
     "mcc_device_free": (ctypes.c_int, [_vp]),
     "mcc_device_pool_clear": (ctypes.c_int, []),

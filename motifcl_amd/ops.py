@@ -138,3 +138,18 @@ def backward_input(grad_out, state, scale, C, in_features, out=None):
         *_buf(grad_out, torch.float32), *_buf(gx, torch.float32),
         batch, in_features, out_features, C))
     return gx
+
+
+def sgd_update(param, grad, lr):
+    """param -= lr * grad in place (sgd_update of MotifCL)."""
+    L = _lib.load()
+    _lib.check(L.mcc_sgd_update_f32(_stream(), *_buf(param, torch.float32), *_buf(grad, torch.float32),
+                                    param.numel(), lr))
+
+
+def adam_update(param, grad, m, v, lr, beta1, beta2, eps, step, weight_decay=0.0):
+    """In-place Adam step with decoupled weight decay (adam_update_fast of MotifCL)."""
+    L = _lib.load()
+    _lib.check(L.mcc_adam_update_f32(_stream(), *_buf(param, torch.float32), *_buf(grad, torch.float32),
+                                     *_buf(m, torch.float32), *_buf(v, torch.float32), param.numel(),
+                                     lr, beta1, beta2, eps, step, weight_decay))

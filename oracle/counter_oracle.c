@@ -358,6 +358,42 @@ void oracle_init_state(const int8_t *tern, uint8_t *state, float *scale, float *
     for (int row = 0; row < out_features; ++row) { scale[row] = s0; v[row] = 0.0f; }
 }
 
+/* ---- FP32 side optimizers: kernels/optim.cl:1-7 and :31-53, host part
+ *      src/ops/optim.cpp:65-86 (bias corrections in binary32) ------------------ */
+void oracle_sgd_update(float *param, const float *grad, size_t n, float lr) {
+    for (size_t i = 0; i < n; ++i) {
+        float d = lr * grad[i];
+        param[i] = param[i] - d;
+    }
+}
+
+void oracle_adam_update(float *param, const float *grad, float *m, float *v, size_t n,
+                        float lr, float beta1, float beta2, float eps, int step,
+                        float weight_decay) {
+    float inv_bias1 = 1.0f / (1.0f - powf(beta1, (float)step));
+    float inv_bias2 = 1.0f / (1.0f - powf(beta2, (float)step));
+    for (size_t i = 0; i < n; ++i) {
+        float g = grad[i];
+        float a = beta1 * m[i];
+        float b = (1.0f - beta1) * g;
+        float mt = a + b;
+        float c = beta2 * v[i];
+        float d = (1.0f - beta2) * g;
+        float e = d * g;
+        float vt = c + e;
+        m[i] = mt;
+        v[i] = vt;
+        float p = param[i];
+        float num = mt * inv_bias1;
+        float den = sqrtf(vt * inv_bias2) + eps;
+        float update = num / den;
+        float s1 = lr * update;
+        float s2 = (lr * weight_decay) * p;
+        float q = p - s1;
+        param[i] = q - s2;
+    }
+}
+
 int oracle_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -65,6 +65,11 @@ def _load():
     lib.oracle_backward_input.argtypes = [_f32p, _u8p, _f32p, _f32p, _c_int, _c_int, _c_int, _c_int]
     lib.oracle_init_state.restype = None
     lib.oracle_init_state.argtypes = [_i8p, _u8p, _f32p, _f32p, _c_int, _c_int, _c_int, _c_float]
+    lib.oracle_sgd_update.restype = None
+    lib.oracle_sgd_update.argtypes = [_f32p, _f32p, ctypes.c_size_t, _c_float]
+    lib.oracle_adam_update.restype = None
+    lib.oracle_adam_update.argtypes = [_f32p, _f32p, _f32p, _f32p, ctypes.c_size_t, _c_float, _c_float,
+                                       _c_float, _c_float, _c_int, _c_float]
     lib.oracle_num_threads.restype = _c_int
     lib.oracle_set_num_threads.argtypes = [_c_int]
     return lib
@@ -198,6 +203,24 @@ def init_state(tern, C, init_gain=1.0):
     _lib.oracle_init_state(tern.ctypes.data_as(_i8p), _u8(state), _f32(scale), _f32(v),
                            C, in_features, out_features, init_gain)
     return state, scale, v
+
+
+def sgd_update(param, grad, lr):
+    """Returns the updated parameter (kernels/optim.cl:1-7)."""
+    p = np.array(param, dtype=np.float32, copy=True).reshape(-1)
+    g = np.ascontiguousarray(grad, dtype=np.float32).reshape(-1)
+    _lib.oracle_sgd_update(_f32(p), _f32(g), p.size, lr)
+    return p.reshape(np.shape(param))
+
+
+def adam_update(param, grad, m, v, lr, beta1, beta2, eps, step, weight_decay=0.0):
+    """Returns (param, m, v) after one Adam step (kernels/optim.cl:31-53, src/ops/optim.cpp:65-86)."""
+    p, mm, vv = (np.array(a, dtype=np.float32, copy=True).reshape(-1) for a in (param, m, v))
+    g = np.ascontiguousarray(grad, dtype=np.float32).reshape(-1)
+    _lib.oracle_adam_update(_f32(p), _f32(g), _f32(mm), _f32(vv), p.size, lr, beta1, beta2, eps, step,
+                            weight_decay)
+    shape = np.shape(param)
+    return p.reshape(shape), mm.reshape(shape), vv.reshape(shape)
 
 
 def num_threads():
