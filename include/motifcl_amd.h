@@ -84,7 +84,10 @@ int mcc_compact_counter_apply_update_dense_batched(
 
 /*
  * Bytes of transient workspace mcc_compact_counter_apply_update_fused needs
- * for the given shape (0 on invalid dimensions).
+ * for the given shape (0 on invalid dimensions): out*in*4 times the number of
+ * token chunks the contraction is split into.  Layers with fewer than about
+ * 1024 output tiles split their tokens so that the whole GPU works on them;
+ * the chunk count depends on (in, out, batch) only.
  */
 size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out_features,
                                                   size_t batch);
@@ -122,9 +125,10 @@ void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
  * CounterStateLinear::apply_update_backward (src/nn/compact_counter.cpp:158-231).
  * The reference's scale_new/denom scratch buffers are not needed; instead the
  * caller lends `workspace`, whose size selects how the step runs:
- *   - >= mcc_compact_counter_fused_workspace_nbytes (a f32[out,in] buffer):
+ *   - >= mcc_compact_counter_fused_workspace_nbytes (one f32[out,in] slice
+ *     per token chunk of the contraction; large layers have one chunk):
  *     contraction into the workspace, then the update kernel.  After the call
- *     the workspace holds grad_w.
+ *     the first out*in floats of the workspace hold grad_w.
  *   - >= mcc_compact_counter_fused_strip_workspace_nbytes but smaller than
  *     the above: the update is applied from the contraction's accumulators
  *     and no weight-sized buffer exists at any time, which is the property

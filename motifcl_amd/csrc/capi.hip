@@ -229,8 +229,11 @@ int mcc_compact_counter_apply_update_dense_batched(void* stream, const mcc_count
 size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out_features,
                                                   size_t batch) {
     if (in_features == 0 || out_features == 0 || batch == 0) return 0;
-    if (out_features > std::numeric_limits<size_t>::max() / sizeof(float) / in_features) return 0;
-    return out_features * in_features * sizeof(float);
+    if (in_features > kIntMax || out_features > kIntMax || batch > kIntMax) return 0;
+    // one f32[out,in] slice per token chunk of the contraction (one chunk for large layers)
+    const size_t slices = mcc::gemm_tn_slices((int)batch, (int)out_features, (int)in_features);
+    if (out_features > std::numeric_limits<size_t>::max() / sizeof(float) / in_features / slices) return 0;
+    return slices * out_features * in_features * sizeof(float);
 }
 
 size_t mcc_compact_counter_fused_strip_workspace_nbytes(size_t in_features, size_t out_features,
@@ -317,7 +320,8 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
     }
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
-        e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features);
+        // the chunk slices start at grad_w: the chunk sums are reduced in place into slice 0
+        e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features, grad_w);
     }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
     {
@@ -345,10 +349,22 @@ int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, co
     if (reinterpret_cast<uintptr_t>(a) % alignof(float) || reinterpret_cast<uintptr_t>(b) % alignof(float) ||
         reinterpret_cast<uintptr_t>(c) % alignof(float))
         return fail(MCC_E_INVALID, "matmul_transpose_a buffers must be 4-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // small outputs split the token range; the chunk products live in a stream-ordered temporary
+    const size_t slices = mcc::gemm_tn_slices((int)k, (int)m, (int)n);
+    float* temp = nullptr;
+    if (slices > 1) {
+        const hipError_t ea = hipMallocAsync(reinterpret_cast<void**>(&temp), slices * m * n * sizeof(float), s);
+        if (ea != hipSuccess) return hip_fail(ea, "matmul_transpose_a could not allocate its chunk buffer");
+    }
     hipError_t e;
     {
-        ScopedKernelTimer timer("gemm_tn_f32", static_cast<hipStream_t>(stream));
-        e = mcc::launch_gemm_tn_f32(static_cast<hipStream_t>(stream), a, b, c, (int)k, (int)m, (int)n);
+        ScopedKernelTimer timer("gemm_tn_f32", s);
+        e = mcc::launch_gemm_tn_f32(s, a, b, c, (int)k, (int)m, (int)n, temp);
+    }
+    if (temp) {
+        const hipError_t ef = hipFreeAsync(temp, s);
+        if (e == hipSuccess) e = ef;
     }
     if (e != hipSuccess) return hip_fail(e, "matmul_transpose_a launch failed");
     return MCC_OK;

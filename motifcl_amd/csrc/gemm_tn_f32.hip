@@ -11,17 +11,25 @@
 namespace mcc {
 namespace {
 
+// Token chunk blockIdx.z of `chunk` tokens goes to slice blockIdx.z of `c` (slices are m*n floats
+// apart); with one chunk this is the whole contraction.
 template <int BM, int BN, bool VEC_A, bool VEC_B>
 __global__ __launch_bounds__(kGemmThreads) void gemm_tn_kernel(const float* __restrict__ a,
                                                                 const float* __restrict__ b,
-                                                                float* __restrict__ c, int K, int M, int N) {
+                                                                float* __restrict__ c, int K, int M, int N,
+                                                                int chunk) {
     using Cfg = TileCfg<BM, BN>;
     __shared__ float lds[Cfg::kLdsFloats];
     const TilePos tp = tile_pos<BM, BN>();
     const int m0 = blockIdx.y * BM;
     const int n0 = blockIdx.x * BN;
+    const int k_begin = blockIdx.z * chunk;
+    const int k_len = K - k_begin < chunk ? K - k_begin : chunk;
+    a += (size_t)k_begin * M;
+    b += (size_t)k_begin * N;
+    c += (size_t)blockIdx.z * M * N;
     floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
-    gemm_tile_mainloop<BM, BN, VEC_A, VEC_B>(a, b, K, M, N, m0, n0, tp, lds, acc);
+    gemm_tile_mainloop<BM, BN, VEC_A, VEC_B>(a, b, k_len, M, N, m0, n0, tp, lds, acc);
 #pragma unroll
     for (int i = 0; i < Cfg::kTilesM; ++i)
 #pragma unroll
@@ -35,26 +43,76 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tn_kernel(const float* __re
         }
 }
 
+// c[e] = ((p0[e] + p1[e]) + p2[e]) + ...: the chunk sums are added in chunk order, so the result
+// does not depend on scheduling.  c may be slice 0 itself.
+__global__ __launch_bounds__(256) void reduce_slices_kernel(const float* __restrict__ slices, float* c, size_t mn,
+                                                           int n_slices) {
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < mn; e += (size_t)gridDim.x * blockDim.x) {
+        float acc = slices[e];
+        for (int s = 1; s < n_slices; ++s) acc = acc + slices[(size_t)s * mn + e];
+        c[e] = acc;
+    }
+}
+
 template <int BM, int BN>
-hipError_t launch_tile(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n) {
-    const dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM);
+hipError_t launch_tile(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n,
+                       const GemmTnPlan& plan) {
+    const dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM, plan.splits);
+    // every chunk starts at a multiple of 16 tokens, so it is as aligned as the matrix itself
     const bool vec_a = (m % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15u) == 0);
     const bool vec_b = (n % 4 == 0) && ((reinterpret_cast<uintptr_t>(b) & 15u) == 0);
     if (vec_a && vec_b)
-        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, true, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m, n);
+        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, true, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m, n,
+                           plan.chunk);
     else if (vec_b)
-        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m, n);
+        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m,
+                           n, plan.chunk);
     else
-        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, false>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m, n);
+        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, false>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m,
+                           n, plan.chunk);
     return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n) {
+// How a contraction is cut up is a function of its shape alone, so that every entry point that
+// contracts the same operands produces the same bits.  Output tiles are 128 x 128 when that
+// already gives 128 tiles, else 64 x 64; the token dimension is split into equal chunks (multiples
+// of 16, at least 256 tokens) until about 1024 workgroups -- four per CU -- exist.  A layer of a
+// 15M-parameter model is 25 tiles: without the split 231 of 256 CUs idle.
+GemmTnPlan plan_gemm_tn(int k, int m, int n) {
+    GemmTnPlan p;
     const long tiles128 = (long)((m + 127) / 128) * ((n + 127) / 128);
-    if (tiles128 >= 128) return launch_tile<128, 128>(stream, a, b, c, k, m, n);
-    return launch_tile<64, 64>(stream, a, b, c, k, m, n);
+    p.tile = tiles128 >= 128 ? 128 : 64;
+    const long tiles = (long)((m + p.tile - 1) / p.tile) * ((n + p.tile - 1) / p.tile);
+    long splits = 1024 / tiles;
+    const long max_splits = k / 256;
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    int chunk = (int)((k + splits - 1) / splits);
+    chunk = (chunk + kBK - 1) / kBK * kBK;
+    p.chunk = chunk;
+    p.splits = (k + chunk - 1) / chunk;
+    return p;
+}
+
+size_t gemm_tn_slices(int k, int m, int n) { return (size_t)plan_gemm_tn(k, m, n).splits; }
+
+// `slices` holds plan.splits * m * n floats when the plan splits the tokens (it may start at c);
+// it is not touched otherwise.
+hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n,
+                              float* slices) {
+    const GemmTnPlan plan = plan_gemm_tn(k, m, n);
+    float* out = plan.splits > 1 ? slices : c;
+    if (plan.splits > 1 && !slices) return hipErrorInvalidValue;
+    hipError_t e = plan.tile == 128 ? launch_tile<128, 128>(stream, a, b, out, k, m, n, plan)
+                                    : launch_tile<64, 64>(stream, a, b, out, k, m, n, plan);
+    if (e != hipSuccess || plan.splits == 1) return e;
+    const size_t mn = (size_t)m * n;
+    const size_t want = (mn + 255) / 256;
+    hipLaunchKernelGGL(reduce_slices_kernel, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, stream, slices,
+                       c, mn, plan.splits);
+    return hipGetLastError();
 }
 
 }  // namespace mcc

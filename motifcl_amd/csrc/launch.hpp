@@ -30,9 +30,18 @@ hipError_t launch_update_dense(hipStream_t stream, uint8_t* state, float* scale,
                                float lr, float lr_scale, float rms_beta, float rms_eps,
                                uint32_t seed);
 
-// c[m,n] = a[k,m]^T . b[k,n]
+// c[m,n] = a[k,m]^T . b[k,n].  Small outputs split the k range into plan.splits chunks whose
+// partial products go to `slices` (plan.splits * m * n floats, may start at c) and are then summed
+// in chunk order into c; gemm_tn_slices tells how many slices a shape needs (1: none).
+struct GemmTnPlan {
+    int tile;    // 128 or 64
+    int splits;  // chunks of the k range
+    int chunk;   // tokens per chunk, a multiple of 16
+};
+GemmTnPlan plan_gemm_tn(int k, int m, int n);
+size_t gemm_tn_slices(int k, int m, int n);
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c,
-                              int k, int m, int n);
+                              int k, int m, int n, float* slices);
 
 // Fused step that keeps G in the contraction's accumulators (counter_fused_strip.hip).
 // Shapes: in_features and out_features multiples of 128; lr_scale == 0 is implied.

@@ -15,10 +15,12 @@ namespace motifcl::nn {
 //          exchange 32 KiB of partial row sums (no weight-sized buffer, as in the reference,
 //          tests/test_memory_truth_gate.cpp:109-113); needs lr_scale == 0 and in/out multiples
 //          of 128, other layers silently use Full
-//   Full   contraction into a f32[out,in] workspace, then the update kernel (a few percent
-//          faster on large layers)
-// Both give identical bytes.
-enum class FusedWorkspace { Strip, Full };
+//   Full   contraction into f32[out,in] workspace slices, then the update kernel (a few percent
+//          faster on large layers; the only way to keep the GPU busy on small ones, whose token
+//          range is split over many workgroups)
+//   Auto   Strip for layers of at least 128 tiles of 128 x 128 (2M weights), Full below
+// All give identical bytes.
+enum class FusedWorkspace { Auto, Strip, Full };
 
 // Ternary finite-state "counter" linear layer trained as a per-synapse automaton: the whole
 // trainable state is a packed 6-bit code per weight plus a per-row scale and a per-row RMS
@@ -69,7 +71,7 @@ private:
     float rms_eps_ = 1e-3f;
     std::uint32_t seed_ = 12345u;
     bool training_ = true;
-    FusedWorkspace fused_workspace_ = FusedWorkspace::Strip;
+    FusedWorkspace fused_workspace_ = FusedWorkspace::Auto;
     std::size_t last_fused_ws_ = 0, last_fused_batch_ = 0;
 };
 

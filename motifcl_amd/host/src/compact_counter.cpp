@@ -106,7 +106,9 @@ void CounterStateLinear::apply_update_backward(const Tensor& grad_out, const Ten
     const std::size_t N = static_cast<std::size_t>(x.shape()[0]);
     const std::size_t in = static_cast<std::size_t>(in_), out = static_cast<std::size_t>(out_);
     std::size_t ws = 0;
-    if (fused_workspace_ == FusedWorkspace::Strip && lr_scale_ == 0.0f)
+    const bool large = ((in + 127) / 128) * ((out + 127) / 128) >= 128;
+    if (lr_scale_ == 0.0f && (fused_workspace_ == FusedWorkspace::Strip ||
+                              (fused_workspace_ == FusedWorkspace::Auto && large)))
         ws = mcc_compact_counter_fused_strip_workspace_nbytes(in, out, N);  // 0: shape not supported
     if (ws == 0) ws = mcc_compact_counter_fused_workspace_nbytes(in, out, N);
     void* scratch = backend_->workspace(ws);

@@ -23,6 +23,7 @@ int main() {
         auto x = Tensor::from_cpu(backend, {N, D}, DType::F32, xh.data());
         auto grad_out = Tensor::from_cpu(backend, {N, D}, DType::F32, gh.data());
         nn::CounterStateLinear layer(backend, D, D, C, 0.003f);
+        layer.set_fused_workspace(nn::FusedWorkspace::Strip);  // the memory-native way at every size
 
         layer.apply_update_backward(grad_out, x, 1u);
         { auto gw = matmul_transpose_a(grad_out, x); layer.apply_update_seed(gw, 1u); }
