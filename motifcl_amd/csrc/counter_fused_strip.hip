@@ -55,6 +55,7 @@ struct StripArgs {
     float* chain;  // [strip][2][128][32]
     int tokens, in_features, out_features;
     int tiles_per_strip, total_tiles;
+    int layer_wgs;  // workgroups the device takes in per residency layer (its CU count)
     unsigned spin_limit;
     Codec cd;
     LutGeom geom;
@@ -210,8 +211,9 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         float* chain = a.chain + (size_t)strip * kStripChainFloats;
 
         floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
-        gemm_tile_mainloop<kTile, kTile, VEC_A, true>(a.grad_out, a.x, a.tokens, a.out_features, a.in_features, m0,
-                                                      n0, tp0, lds, acc);
+        // even progress of the workgroups that share a CU: a strip is as slow as its slowest tile
+        gemm_tile_mainloop<kTile, kTile, VEC_A, true, true>(a.grad_out, a.x, a.tokens, a.out_features, a.in_features,
+                                                            m0, n0, tp0, lds, acc, (int)blockIdx.x / a.layer_wgs);
 
         park_accumulators(acc);
         // the hand-off sequence is latency-bound and other workgroups of this CU are still in
@@ -425,8 +427,12 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kGemmThreads, 0);
     if (err != hipSuccess) return err;
     const long capacity = (long)cus * per_cu;
+    a.layer_wgs = cus;
     if (capacity < a.tiles_per_strip) return hipErrorLaunchOutOfResources;
-    const int grid = (int)(capacity < a.total_tiles ? capacity : a.total_tiles);
+    // a whole number of strips per pass of the persistent grid: a strip that straddled two passes
+    // would park its early tiles' workgroups for the length of a pass
+    const long whole = capacity / a.tiles_per_strip * a.tiles_per_strip;
+    const int grid = (int)(whole < a.total_tiles ? whole : a.total_tiles);
 
     const int clear_words = (int)((kHeaderBytes + flags_bytes((size_t)strips)) / sizeof(int));
     hipLaunchKernelGGL(strip_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, stream,

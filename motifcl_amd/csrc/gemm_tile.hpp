@@ -73,11 +73,29 @@ __device__ __forceinline__ TilePos tile_pos() {
 // TileCfg::kLdsFloats floats.  Ends with a barrier, so lds may be reused right after.
 // Accumulator layout (v_mfma_f32_32x32x2_f32): acc[i][j][r] is row
 // wm0 + 32 i + 8 (r/4) + 4 half + r%4 and column wn0 + 32 j + l32 of the tile.
-template <int BM, int BN, bool VEC_A, bool VEC_B>
+//
+// ROTATE_PRIORITY: the hardware issues from a SIMD's oldest wave first, so of the four workgroups
+// resident on a CU the first one runs up to 30 % ahead of the last.  Kernels whose workgroups wait
+// for each other want even progress instead: every kPriorityPeriod slabs the wave moves to the
+// next of four priority levels, and workgroups resident together start at different levels
+// (priority_phase = the workgroup's residency layer), so each leads a quarter of the time.
+constexpr int kPriorityPeriod = 16;
+
+__device__ __forceinline__ void set_wave_priority(int level) {
+    switch (level) {  // s_setprio takes an immediate
+        case 0: __builtin_amdgcn_s_setprio(0); break;
+        case 1: __builtin_amdgcn_s_setprio(1); break;
+        case 2: __builtin_amdgcn_s_setprio(2); break;
+        default: __builtin_amdgcn_s_setprio(3); break;
+    }
+}
+
+template <int BM, int BN, bool VEC_A, bool VEC_B, bool ROTATE_PRIORITY = false>
 __device__ __forceinline__ void gemm_tile_mainloop(const float* __restrict__ a, const float* __restrict__ b,
                                                    int K, int M, int N, int m0, int n0, const TilePos& tp,
                                                    float* lds,
-                                                   floatx16 (&acc)[TileCfg<BM, BN>::kTilesM][TileCfg<BM, BN>::kTilesN]) {
+                                                   floatx16 (&acc)[TileCfg<BM, BN>::kTilesM][TileCfg<BM, BN>::kTilesN],
+                                                   int priority_phase = 0) {
     using Cfg = TileCfg<BM, BN>;
     float* lds_a = lds;
     float* lds_b = lds + kBK * Cfg::kLdA;
@@ -120,6 +138,8 @@ __device__ __forceinline__ void gemm_tile_mainloop(const float* __restrict__ a, 
 
     fetch(0);
     for (int k0 = 0; k0 < K; k0 += kBK) {
+        if (ROTATE_PRIORITY && (k0 & (kPriorityPeriod * kBK - 1)) == 0)
+            set_wave_priority((k0 / (kPriorityPeriod * kBK) + priority_phase) & 3);
         stage();
         __syncthreads();
         if (k0 + kBK < K) fetch(k0 + kBK);
