@@ -97,7 +97,7 @@ def time_steps(step_fn, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def bench_fused(L, ops, name, steps, warmup, fused_path="workspace"):
+def bench_fused(L, ops, name, steps, warmup, fused_path="workspace", graph=False):
     import torch
     desc, shapes, layers, tokens = WORKLOADS[name]
     gen = torch.Generator(device="cuda")
@@ -129,6 +129,20 @@ def bench_fused(L, ops, name, steps, warmup, fused_path="workspace"):
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
+    graph_ms = None
+    if graph:
+        # the same step captured once and replayed: what a launch-bound small model gains when the
+        # host submits one graph instead of 3 launches per tensor (the seeds are baked in, so this
+        # is a launch-cost measurement, not a training loop)
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            step(0)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                step(0)
+        torch.cuda.synchronize()
+        graph_ms = time_steps(lambda i: g.replay(), steps, 2)
     L.mcc_profiler_reset()
     L.mcc_profiler_enable(1)
     ms_per_step = time_steps(step, steps, 0)
@@ -155,7 +169,7 @@ def bench_fused(L, ops, name, steps, warmup, fused_path="workspace"):
                      "launches": gemm_n, "avg_launch_ms": gemm_ms / max(gemm_n, 1),
                      "algorithmic_flops_per_step": flops},
         "kernel_ms_per_step": {kernel: gemm_ms / steps, "counter_update": upd_ms / steps},
-        "fused_path": fused_path, "workspace_bytes": ws_bytes,
+        "fused_path": fused_path, "workspace_bytes": ws_bytes, "graph_replay_ms_per_step": graph_ms,
     }
     sample = tensors[0]
     del ws
@@ -362,6 +376,9 @@ def main():
     ap.add_argument("--fused-path", default="workspace", choices=["workspace", "strip"],
                     help="workspace: contraction into a lent f32[out,in] buffer, then the update kernel; "
                          "strip: update applied from the contraction's accumulators, no weight-sized buffer")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the fused step captured into a HIP graph and replayed (reported beside "
+                         "the eager figure, which stays the headline)")
     ap.add_argument("--no-update-only", action="store_true", help="skip the cfg3 update-only leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -391,7 +408,7 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
-    fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup, args.fused_path)
+    fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup, args.fused_path, args.graph)
     line = {
         "metric": "counter-synapse updates/s (Gparam/s)",
         "value": fused["value"], "unit": "Gparam/s", "n_gpus": 1, "steps": args.steps,
@@ -400,6 +417,7 @@ def main():
         "config": fused["config"], "roofline": fused["roofline"],
         "kernel_ms_per_step": fused["kernel_ms_per_step"],
         "fused_path": fused["fused_path"], "fused_workspace_bytes": fused["workspace_bytes"],
+        "graph_replay_ms_per_step": fused["graph_replay_ms_per_step"],
         "device": L.mcc_device_name().decode(),
     }
     if not args.no_cpu:
