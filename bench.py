@@ -291,7 +291,7 @@ def bench_update_only(L, ops, steps, warmup):
                      "algorithmic_bytes_per_launch": BYTES_PER_PARAM * params},
     }
     sample = tensors[0]
-    return out, sample
+    return out, sample, tensors
 
 
 def cpu_baseline_fused(sample, tokens, rows, min_seconds=8.0):
@@ -367,6 +367,63 @@ def parity_leg(ops):
     }
 
 
+def parity_full_size_fused(ops, tokens=32768):
+    """Size-independent properties at the cfg4 shapes: the two fused implementations (two-kernel and
+    accumulator-resident) give the same bytes, and sampled rows of the contraction agree with a
+    double-precision product."""
+    import torch
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    out = {"tokens": tokens, "shapes": []}
+    for (n_out, n_in) in [(4096, 4096), (11008, 4096), (4096, 11008)]:
+        x = torch.randn(tokens, n_in, device="cuda", generator=gen)
+        dy = torch.randn(tokens, n_out, device="cuda", generator=gen) * 0.01
+        st0 = make_state(gen, n_out, n_in)
+        results = []
+        ws_full = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, tokens), dtype=torch.uint8, device="cuda")
+        ws_strip = torch.empty(ops.fused_strip_workspace_nbytes(n_in, n_out, tokens), dtype=torch.uint8, device="cuda")
+        for ws in (ws_full, ws_strip):
+            d = [t.clone() for t in st0]
+            ops.apply_update_fused(d[0], d[1], d[2], dy, x, ws, C, LR, LR_SCALE, BETA, EPS, 4242)
+            ops.fused_check(ws, n_in, n_out, tokens)
+            results.append(d)
+        same = all(torch.equal(a, b) for a, b in zip(*results))
+        rows = torch.arange(0, n_out, max(1, n_out // 8), device="cuda")[:8]
+        g = ws_full.view(torch.float32)[: n_out * n_in].view(n_out, n_in)[rows].double()
+        ref = dy[:, rows].double().t() @ x.double()
+        rel = float((g - ref).abs().max() / ref.abs().max())
+        changed = float((results[0][0] != st0[0]).float().mean())
+        out["shapes"].append({"out": n_out, "in": n_in, "two_kernel_equals_accumulator_resident": bool(same),
+                              "max_abs_dG_over_max_abs_G_vs_f64_on_8_rows": rel,
+                              "state_bytes_changed_fraction": changed})
+        del x, dy, ws_full, ws_strip, results, g, ref
+        torch.cuda.empty_cache()
+    return out
+
+
+def parity_full_size_update_only(ops, tensors, picks=(0, 4, 6, 117, 223)):
+    """cfg3 at full size: a sample of the 224 tensors, each updated on the GPU by the batched call
+    and on the CPU by the oracle from the same snapshot; bytes must be identical."""
+    import numpy as np
+    import torch
+    from oracle import counter_oracle as oracle
+    picks = [k for k in picks if k < len(tensors)]
+    before = {k: [t.cpu().numpy().copy() for t in tensors[k][0]] for k in picks}
+    batch = ops.UpdateBatch([(st[0], st[1], st[2], g) for (st, g, _, _) in tensors], LR,
+                            [777 + k for k in range(len(tensors))])
+    ops.apply_update_dense_batched(batch, C, LR_SCALE, BETA, EPS)
+    torch.cuda.synchronize()
+    ok = []
+    for k in picks:
+        (st, g, n_out, n_in) = tensors[k]
+        exp = oracle.update_dense(before[k][0], before[k][1], before[k][2], g.cpu().numpy(), C, LR, LR_SCALE,
+                                  BETA, EPS, 777 + k)
+        got = [t.cpu().numpy() for t in st]
+        ok.append(bool(all(np.array_equal(a, b) for a, b in zip(got, exp))))
+    return {"sampled_tensor_indices": picks, "shapes": [[tensors[k][2], tensors[k][3]] for k in picks],
+            "state_scale_v_bit_exact": ok, "all_bit_exact": bool(all(ok))}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -423,6 +480,8 @@ def main():
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_fused(fused_sample, tokens, args.cpu_rows)
         line["parity"] = parity_leg(ops)
+        if args.workload == "cfg4":
+            line["parity"]["full_size"] = parity_full_size_fused(ops)
     del fused_sample
     torch.cuda.empty_cache()
     line["side_optimizer"] = bench_side_optimizer(L, ops, max(3, args.steps), 2)
@@ -430,9 +489,11 @@ def main():
     line["layer_products"] = bench_layer_products(L, ops, args.workload, max(2, args.steps // 2), 1)
     torch.cuda.empty_cache()
     if not args.no_update_only:
-        uo, uo_sample = bench_update_only(L, ops, args.steps, args.warmup)
+        uo, uo_sample, uo_tensors = bench_update_only(L, ops, args.steps, args.warmup)
         if not args.no_cpu:
             uo["cpu_baseline"] = cpu_baseline_dense(uo_sample)
+            uo["parity_full_size"] = parity_full_size_update_only(ops, uo_tensors)
+        del uo_tensors
         line["update_only"] = uo
     print(json.dumps(line))
 
