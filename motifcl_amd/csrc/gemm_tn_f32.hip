@@ -13,13 +13,13 @@ namespace {
 
 // Token chunk blockIdx.z of `chunk` tokens goes to slice blockIdx.z of `c` (slices are m*n floats
 // apart); with one chunk this is the whole contraction.
-template <int BM, int BN, bool VEC_A, bool VEC_B>
+template <int BM, int BN, bool VEC_A, bool VEC_B, bool DIRECT>
 __global__ __launch_bounds__(kGemmThreads) void gemm_tn_kernel(const float* __restrict__ a,
                                                                 const float* __restrict__ b,
                                                                 float* __restrict__ c, int K, int M, int N,
                                                                 int chunk) {
     using Cfg = TileCfg<BM, BN>;
-    __shared__ float lds[Cfg::kLdsFloats];
+    __shared__ float lds[DIRECT ? DirectCfg<BM, BN>::kLdsFloats : Cfg::kLdsFloats];
     const TilePos tp = tile_pos<BM, BN>();
     const int m0 = blockIdx.y * BM;
     const int n0 = blockIdx.x * BN;
@@ -29,7 +29,10 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tn_kernel(const float* __re
     b += (size_t)k_begin * N;
     c += (size_t)blockIdx.z * M * N;
     floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
-    gemm_tile_mainloop<BM, BN, VEC_A, VEC_B>(a, b, k_len, M, N, m0, n0, tp, lds, acc);
+    if (DIRECT)
+        gemm_tile_mainloop_direct<BM, BN>(a, b, k_len, M, N, m0, n0, tp, lds, acc);
+    else
+        gemm_tile_mainloop<BM, BN, VEC_A, VEC_B>(a, b, k_len, M, N, m0, n0, tp, lds, acc);
 #pragma unroll
     for (int i = 0; i < Cfg::kTilesM; ++i)
 #pragma unroll
@@ -61,15 +64,20 @@ hipError_t launch_tile(hipStream_t stream, const float* a, const float* b, float
     // every chunk starts at a multiple of 16 tokens, so it is as aligned as the matrix itself
     const bool vec_a = (m % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15u) == 0);
     const bool vec_b = (n % 4 == 0) && ((reinterpret_cast<uintptr_t>(b) & 15u) == 0);
-    if (vec_a && vec_b)
-        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, true, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m, n,
-                           plan.chunk);
+    // whole tiles and whole slabs (every chunk is a multiple of 16 tokens when k is): direct-to-LDS
+    const bool direct = vec_a && vec_b && m % BM == 0 && n % BN == 0 && k % kBK == 0;
+    if (direct)
+        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, true, true, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k,
+                           m, n, plan.chunk);
+    else if (vec_a && vec_b)
+        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, true, true, false>), grid, dim3(kGemmThreads), 0, stream, a, b, c,
+                           k, m, n, plan.chunk);
     else if (vec_b)
-        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m,
-                           n, plan.chunk);
+        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, true, false>), grid, dim3(kGemmThreads), 0, stream, a, b, c,
+                           k, m, n, plan.chunk);
     else
-        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, false>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k, m,
-                           n, plan.chunk);
+        hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, false, false>), grid, dim3(kGemmThreads), 0, stream, a, b,
+                           c, k, m, n, plan.chunk);
     return hipGetLastError();
 }
 
