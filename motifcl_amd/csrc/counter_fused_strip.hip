@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         tc.neg_lim_neg = -(float)a.geom.lim_neg;
         tc.lim_pos = (float)a.geom.lim_pos;
         tc.two_m24 = 1.0f / 16777216.0f;
-        tc.seed = a.seed;
+        tc.seed_mix = seed_mix(a.seed);
         // 32-bit byte offsets from the state base (the launch checks that the state is smaller
         // than 2 GiB): one add per element on top of a per-thread part
         const uint32_t row_bytes = 3u * (uint32_t)groups_per_row;

@@ -35,6 +35,25 @@ MCC_HD uint32_t hash_rest(uint32_t x) {
 
 MCC_HD uint32_t hash_u32(uint32_t x) { return hash_rest(hash_first(x)); }
 
+// hash_rest without its last xor-shift: hash_rest(x) == u ^ (u >> 16) with u = hash_open(x).
+MCC_HD uint32_t hash_open(uint32_t x) {
+    x *= 0x7feb352du;
+    x ^= x >> 15;
+    x *= 0x846ca68bu;
+    return x;
+}
+
+// The draw of kernels/compact_counter.cl:127 is hash(seed ^ hash(elem)).  With h = u ^ (u >> 16)
+// the inner hash and y = seed ^ h, the outer hash starts with y ^ (y >> 16), and
+//   y >> 16 = (seed >> 16) ^ (h >> 16) = (seed >> 16) ^ (u >> 16)        ((u >> 16) >> 16 == 0)
+//   y ^ (y >> 16) = seed ^ u ^ (u >> 16) ^ (seed >> 16) ^ (u >> 16) = (seed ^ (seed >> 16)) ^ u
+// so the inner hash's last step, the xor with the seed and the outer hash's first step collapse
+// into one xor with a per-tensor constant.
+MCC_HD uint32_t seed_mix(uint32_t seed) { return seed ^ (seed >> 16); }
+
+// hash_u32(seed ^ hash_rest(x)) given mix = seed_mix(seed)
+MCC_HD uint32_t draw_hash(uint32_t mix, uint32_t x) { return hash_rest(mix ^ hash_open(x)); }
+
 // 24-bit word of one packed group -> code k (kernels/compact_counter.cl:25-31)
 MCC_HD uint32_t code_of(uint32_t word, int k) { return (word >> (6 * k)) & 0x3fu; }
 
@@ -185,7 +204,7 @@ struct TickConsts {
     float neg_lr;     // -lr
     float neg_lim_neg, lim_pos;  // clamp of floor(val), as floats
     float two_m24;               // 2^-24 (kept in a register: see the kernel)
-    uint32_t seed;
+    uint32_t seed_mix;           // seed_mix(seed)
 };
 
 // One stochastic-rounding tick (kernels/compact_counter.cl:120-136).
@@ -200,7 +219,7 @@ MCC_HD uint32_t tick_code(uint32_t code, float gw, const TickConsts& tc, uint32_
     const float val = c_reb[code] + tick;
     const float f = floorf(val);
     const float frac = val - f;
-    const uint32_t h = hash_u32(tc.seed ^ hash_rest(elem_x));
+    const uint32_t h = draw_hash(tc.seed_mix, elem_x);
     const float rnd = (float)(h & 0x00ffffffu) * tc.two_m24;
     // q_off + floor + [rnd < frac]: one add-with-carry on the GPU
     const int idx = q_off[code] + (int)clamp_f(f, tc.neg_lim_neg, tc.lim_pos) + (rnd < frac ? 1 : 0);

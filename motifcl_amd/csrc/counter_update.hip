@@ -154,7 +154,7 @@ __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTen
     rc.tc.neg_lr = -t.lr;
     rc.tc.neg_lim_neg = -(float)a.geom.lim_neg;
     rc.tc.lim_pos = (float)a.geom.lim_pos;
-    rc.tc.seed = t.seed;
+    rc.tc.seed_mix = seed_mix(t.seed);
     rc.tc.two_m24 = 1.0f / 16777216.0f;
     // v_mul_f32 issues at twice the rate when both operands are VGPRs: keep the per-row
     // multipliers out of scalar registers and literals
@@ -407,7 +407,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
                 tc.neg_lr = -t.lr;
                 tc.neg_lim_neg = -(float)a.geom.lim_neg;
                 tc.lim_pos = (float)a.geom.lim_pos;
-                tc.seed = t.seed;
+                tc.seed_mix = seed_mix(t.seed);
                 tc.two_m24 = 1.0f / 16777216.0f;
                 sh.tc = tc;
                 sh.fast_div = row_takes_fast_division(rs.denom, g_sq, min_key) ? 1 : 0;

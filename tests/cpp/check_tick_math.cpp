@@ -41,7 +41,7 @@ int main(int argc, char** argv) {
             mcc::TickConsts tc;
             tc.dn = dn; tc.r = 1.0f / dn; tc.k = cd.Cf / s_new; tc.neg_lr = -lr;
             tc.neg_lim_neg = -(float)g.lim_neg; tc.lim_pos = (float)g.lim_pos;
-            tc.seed = seed; tc.two_m24 = 1.0f / 16777216.0f;
+            tc.seed_mix = mcc::seed_mix(seed); tc.two_m24 = 1.0f / 16777216.0f;
             for (uint32_t code = 0; code < 64; ++code) c_reb[code] = mcc::c_reb_entry(code, cd, s_old / s_new);
             return tc;
         };
@@ -95,6 +95,14 @@ int main(int argc, char** argv) {
                 ++checked;
                 if ((int)got != exp) { if (mismatches < 10) std::printf("TABLE MISMATCH C=%d code=%d g=%d got=%u exp=%d\n", C, code, gi, got, exp); ++mismatches; }
             }
+    }
+    // collapsed seed xor: hash(seed ^ hash(elem)) == hash_rest(seed_mix(seed) ^ hash_open(hash_first(elem)))
+    for (int i = 0; i < 4000000; ++i) {
+        const uint32_t seed = (uint32_t)next_u64(), elem = (uint32_t)next_u64();
+        if (mcc::draw_hash(mcc::seed_mix(seed), mcc::hash_first(elem)) != mcc::hash_u32(seed ^ mcc::hash_u32(elem))) {
+            std::printf("draw_hash differs at seed=%u elem=%u\n", seed, elem);
+            return 2;
+        }
     }
     // shared first hash step: (e + k) ^ ((e + k) >> 16) == (e ^ (e >> 16)) ^ k for e % 4 == 0
     for (long it = 0; it < 4000000; ++it) {
