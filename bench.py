@@ -36,9 +36,9 @@ BYTES_PER_PARAM = 5.5          # 4 (read G) + 0.75 (read state) + 0.75 (write st
 # 1 GiB copy; summaries and commands under profiles/).  They are reported, not re-measured
 # here, and only for the default workloads they were measured on.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg4/gemm_tn_f32": 24.76e9,      # average over the 7 launches of a step (algorithmic 1.4 GB)
-    "cfg4/fused_strip": 28.18e9,      # average over the 7 launches of a step, --fused-path strip
-    "cfg3/update_rows": 36.15e9,      # the batched call of a step (algorithmic 35.64 GB)
+    "cfg4/gemm_tn_f32": 24.90e9,      # average over the 7 launches of a step (algorithmic 1.4 GB)
+    "cfg4/fused_strip": 27.50e9,      # average over the 7 launches of a step, --fused-path strip
+    "cfg3/update_rows": 36.17e9,      # the batched call of a step (algorithmic 35.64 GB)
 }
 
 
