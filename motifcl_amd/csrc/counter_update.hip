@@ -363,7 +363,28 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
             q[jj] = g_row[gc];
             words[jj] = load_group_dword(s_row + 3u * gc);
         }
-        // running sums travel wave 0 -> 1 -> ... -> W-1 in iteration order
+        // What does not depend on the order happens before the hand-off, in all waves at once: the
+        // squares, the products with t, and the minimum of the magnitude keys (a minimum may be
+        // taken in any order).  Only the additions travel wave 0 -> 1 -> ... -> W-1.  (Long
+        // per-wave stretches have no registers to spare for the squares and do it all in turn.)
+        constexpr bool kPre = J <= 11;
+        float sq[kPre ? J : 1][4], gt[kPre && WITH_GS ? J : 1][4];
+        uint32_t my_key = 0xffffffffu;
+        if (kPre) {
+#pragma unroll
+            for (int jj = 0; jj < J; ++jj) {
+                const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+                const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
+                                    live ? q[jj].w : 0.0f};
+                my_key = umin3(my_key, range_key(g[0]), range_key(g[1]));
+                my_key = umin3(my_key, range_key(g[2]), range_key(g[3]));
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    sq[jj][k] = g[k] * g[k];
+                    if (WITH_GS) gt[jj][k] = g[k] * (float)(code_q(code_of(words[jj], k), a.cd) - 1);
+                }
+            }
+        }
         RowAcc acc;
 #pragma unroll
         for (int step = 0; step < W; ++step) {
@@ -373,12 +394,23 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
                     acc.grad_s = sh.part_gs[lane];
                     acc.min_key = sh.part_key[lane];
                 }
+                if (kPre) {
+                    acc.min_key = umin(acc.min_key, my_key);
 #pragma unroll
-                for (int jj = 0; jj < J; ++jj) {
-                    const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
-                    const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
-                                        live ? q[jj].w : 0.0f};
-                    accumulate<WITH_GS>(acc, g, words[jj], a.cd);
+                    for (int jj = 0; jj < J; ++jj)
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            acc.g_sq = acc.g_sq + sq[jj][k];
+                            if (WITH_GS) acc.grad_s = acc.grad_s + gt[jj][k];
+                        }
+                } else {
+#pragma unroll
+                    for (int jj = 0; jj < J; ++jj) {
+                        const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+                        const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
+                                            live ? q[jj].w : 0.0f};
+                        accumulate<WITH_GS>(acc, g, words[jj], a.cd);
+                    }
                 }
                 if (step < W - 1) {
                     sh.part_sq[lane] = acc.g_sq;
