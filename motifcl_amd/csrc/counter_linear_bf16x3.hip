@@ -1,0 +1,400 @@
+// Forward and input-gradient products of the counter layer on the bf16 matrix cores, with fp32
+// accuracy.
+//
+// The weight is W[o,i] = scale[o] * t[o,i] with t a small integer (-1, 0, 1 for every reachable
+// code), and a small integer is exact in bf16.  A binary32 activation is the exact sum of three
+// bf16 numbers,
+//     x = hi + mid + lo,   hi = bf16(x),  mid = bf16(x - hi),  lo = bf16(x - hi - mid)
+// (each subtraction is exact: 24 significant bits are peeled off 8 at a time; only numbers within
+// 2^16 of the smallest normal lose their tail), and a bf16 x bf16 product is exact in binary32.
+// So
+//     sum_k x[k] * t[k] = sum_k hi[k] t[k] + sum_k mid[k] t[k] + sum_k lo[k] t[k]
+// is three bf16 MFMA passes into one fp32 accumulator whose every product is exact: the same
+// mathematical terms as an fp32 contraction, summed in another order, at 16 x the matrix rate
+// per pass (v_mfma_f32_32x32x16_bf16 against v_mfma_f32_32x32x2_f32).
+//   forward         y[r,o]      = scale[o] * sum_i x[r,i] * t[o,i]
+//   backward_input  grad_x[r,i] = sum_o (grad_out[r,o] * scale[o]) * t[o,i]
+// (kernels/vulkan/counter_forward_f32_rb4.comp, counter_backward_input_f32_rb4.comp; the second
+// line multiplies by the scale first, as kernels/compact_counter.cl:262-267 does).  Non-finite
+// activations are outside this kernel's contract (inf - inf in the split).
+//
+// Tile: 128 x 128 per workgroup of 4 waves (2 x 2, 64 x 64 each), 32-deep slabs.  LDS holds the
+// three activation planes and the weight tile as [row][32 bf16] = 64-byte rows whose four
+// 16-byte chunks are XOR-swizzled with bits 1-2 of the row, which makes the 16-byte MFMA operand
+// reads (lane = row, 8 consecutive k) conflict-free without padding: 32 KiB per workgroup.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "counter_math.hpp"
+#include "gemm_tile.hpp"
+#include "launch.hpp"
+
+namespace mcc {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kT = 128;        // tile rows and columns
+constexpr int kK = 32;         // slab depth
+constexpr int kRowBytes = 64;  // 32 bf16
+constexpr int kPlaneBytes = kT * kRowBytes;
+
+struct Lin3Args {
+    const float* act;      // [rows, K]
+    const uint8_t* state;  // packed [out, in/4 * 3]
+    const float* scale;    // [out]
+    float* c;              // [rows, N]
+    Codec cd;
+    int rows, in_features, out_features;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    const bf16x2 p = {(__bf16)a, (__bf16)b};  // round to nearest even
+    return __builtin_bit_cast(uint32_t, p);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t p) { return __uint_as_float(p << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
+
+// Byte offset of 8-byte piece `half` of 16-byte chunk `chunk` of row `row` in a swizzled tile.
+__device__ __forceinline__ int tile_offset(int row, int chunk, int half) {
+    return row * kRowBytes + ((chunk ^ ((row >> 1) & 3)) << 4) + (half << 3);
+}
+
+// Splits four activations into their three bf16 planes and stores each as 8 bytes.
+__device__ __forceinline__ void store_split(uint8_t* planes, int offset, float x0, float x1, float x2, float x3) {
+    const uint32_t h01 = pack_bf16(x0, x1), h23 = pack_bf16(x2, x3);
+    const float r0 = x0 - bf16_lo(h01), r1 = x1 - bf16_hi(h01), r2 = x2 - bf16_lo(h23), r3 = x3 - bf16_hi(h23);
+    const uint32_t m01 = pack_bf16(r0, r1), m23 = pack_bf16(r2, r3);
+    const float s0 = r0 - bf16_lo(m01), s1 = r1 - bf16_hi(m01), s2 = r2 - bf16_lo(m23), s3 = r3 - bf16_hi(m23);
+    const uint32_t l01 = pack_bf16(s0, s1), l23 = pack_bf16(s2, s3);
+    *reinterpret_cast<uint2*>(planes + offset) = make_uint2(h01, h23);
+    *reinterpret_cast<uint2*>(planes + kPlaneBytes + offset) = make_uint2(m01, m23);
+    *reinterpret_cast<uint2*>(planes + 2 * kPlaneBytes + offset) = make_uint2(l01, l23);
+}
+
+__device__ __forceinline__ uint32_t fetch_group(const uint8_t* state, size_t group, size_t last_group, bool valid) {
+    if (!valid) return 0xffffffffu;  // marks "no weight": decoded to zero below
+    const uint8_t* p = state + 3 * group;
+    if (group == last_group) return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+    uint32_t w;
+    __builtin_memcpy(&w, p, 4);
+    return w & 0x00ffffffu;
+}
+
+// t = code / lv - 1 of code k of a packed word, as a float (0 for the "no weight" marker).
+__device__ __forceinline__ float ternary_of(uint32_t word, int k, const Codec& cd) {
+    const float t = (float)(code_q(code_of(word, k), cd) - 1);
+    return word == 0xffffffffu ? 0.0f : t;
+}
+
+__device__ __forceinline__ bf16x8 read_operand(const uint8_t* tile, int row, int chunk) {
+    const uint4 v = *reinterpret_cast<const uint4*>(tile + tile_offset(row, chunk, 0));
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+// Whole tiles and whole slabs (rows, N multiples of 128, K a multiple of 32, 16-byte aligned
+// activation and scale, buffers below 4 GiB): nothing is checked, every address is a per-thread
+// 32-bit offset computed once plus a per-slab constant.
+template <bool FORWARD>
+__global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_kernel(Lin3Args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * kPlaneBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[kPlaneBytes];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, kh = lane >> 5;
+    const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+    const int m0 = blockIdx.y * kT, n0 = blockIdx.x * kT;
+    const int K = FORWARD ? a.in_features : a.out_features;
+    const int N = FORWARD ? a.out_features : a.in_features;
+    const uint32_t gpr = (uint32_t)a.in_features >> 2;
+    const uint32_t last_off = 3u * ((uint32_t)a.out_features * gpr - 1u);
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // thread (row = tid / 8 + 32 p, c4 = tid % 8) stages 4 activations per p; byte offsets
+    const int c4 = tid & 7, row0 = tid >> 3;
+    uint32_t off_a[4], off_w[4];
+    int lds_off_a[4], lds_off_b[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int row = row0 + 32 * p;
+        off_a[p] = ((uint32_t)(m0 + row) * (uint32_t)K + 4u * c4) * 4u;
+        lds_off_a[p] = tile_offset(row, c4 >> 1, c4 & 1);
+        if (FORWARD) {
+            // (weight row n = row, group c4 of the slab)
+            off_w[p] = 3u * ((uint32_t)(n0 + row) * gpr + (uint32_t)c4);
+            lds_off_b[p] = lds_off_a[p];
+        } else {
+            // (weight rows k = 4 oq + p with oq = tid % 8, group g = tid / 8 of the tile's columns)
+            off_w[p] = 3u * ((uint32_t)(4 * c4 + p) * gpr + (uint32_t)(n0 >> 2) + (uint32_t)row0);
+            lds_off_b[p] = tile_offset(4 * row0 + p, c4 >> 1, c4 & 1);  // column n = 4 g + p, k = 4 oq ..
+        }
+    }
+    const uint32_t w_step = FORWARD ? 3u * (kK / 4) : 3u * kK * gpr;  // packed bytes per slab
+
+    float4 ra[4];
+    uint32_t rw[4];
+    auto fetch = [&](int k0, uint32_t w_base) {
+        float4 sc = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (!FORWARD) sc = *reinterpret_cast<const float4*>(a.scale + k0 + 4 * c4);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const float4 x = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.act) + off_a[p] +
+                                                              4u * (uint32_t)k0);
+            // (grad_out * scale) first, as the reference does
+            ra[p] = FORWARD ? x : make_float4(x.x * sc.x, x.y * sc.y, x.z * sc.z, x.w * sc.w);
+            // one 4-byte load per packed group; the tensor's last group has no byte after it and
+            // is fetched one byte early
+            const uint32_t off = off_w[p] + w_base;
+            const uint32_t is_last = off == last_off ? 1u : 0u;
+            uint32_t w;
+            __builtin_memcpy(&w, a.state + (off - is_last), 4);
+            rw[p] = w >> (8 * is_last);
+        }
+    };
+    auto ternary = [&](uint32_t word, int k) { return (float)(code_q(code_of(word, k), a.cd) - 1); };
+    auto stage = [&]() {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) store_split(lds_a, lds_off_a[p], ra[p].x, ra[p].y, ra[p].z, ra[p].w);
+        if (FORWARD) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const uint32_t lo = pack_bf16(ternary(rw[p], 0), ternary(rw[p], 1));
+                const uint32_t hi = pack_bf16(ternary(rw[p], 2), ternary(rw[p], 3));
+                *reinterpret_cast<uint2*>(lds_b + lds_off_b[p]) = make_uint2(lo, hi);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {  // rw[r] is weight row k = 4 oq + r; column 4 g + j takes code j of each
+                const uint32_t lo = pack_bf16(ternary(rw[0], j), ternary(rw[1], j));
+                const uint32_t hi = pack_bf16(ternary(rw[2], j), ternary(rw[3], j));
+                *reinterpret_cast<uint2*>(lds_b + lds_off_b[j]) = make_uint2(lo, hi);
+            }
+        }
+    };
+    int read_a[2], read_b[2];  // operand read offsets for chunk kh; the chunk of step s is 2 s + kh
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        read_a[i] = wm0 + 32 * i + l32;
+        read_b[i] = wn0 + 32 * i + l32;
+    }
+
+    uint32_t w_base = 0;
+    fetch(0, 0);
+    for (int k0 = 0; k0 < K; k0 += kK) {
+        stage();
+        __syncthreads();
+        w_base += w_step;
+        if (k0 + kK < K) fetch(k0 + kK, w_base);
+#pragma unroll
+        for (int s = 0; s < kK / 16; ++s) {
+            const int chunk = 2 * s + kh;
+            bf16x8 fb[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb[j] = read_operand(lds_b, read_b[j], chunk);
+#pragma unroll
+            for (int plane = 0; plane < 3; ++plane) {
+                bf16x8 fa[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) fa[i] = read_operand(lds_a + plane * kPlaneBytes, read_a[i], chunk);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wn0 + 32 * j + l32;
+            const float s = FORWARD ? a.scale[col] : 1.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm0 + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+                a.c[(size_t)row * N + col] = FORWARD ? acc[i][j][r] * s : acc[i][j][r];
+            }
+        }
+}
+
+// Any shape: every access is checked and short slabs are zero-filled.
+template <bool FORWARD, bool VEC_A>
+__global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_edge_kernel(Lin3Args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * kPlaneBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[kPlaneBytes];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, kh = lane >> 5;
+    const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+    const int m0 = blockIdx.y * kT, n0 = blockIdx.x * kT;
+    const int K = FORWARD ? a.in_features : a.out_features;
+    const int N = FORWARD ? a.out_features : a.in_features;
+    const int gpr = a.in_features >> 2;
+    const size_t last_group = (size_t)a.out_features * gpr - 1;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // staging registers of one slab: 4 float4 of activation and 4 packed groups per thread
+    float4 ra[4];
+    uint32_t rw[4];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int idx = tid + kGemmThreads * p;
+            const int row = idx >> 3, c4 = idx & 7;
+            float4 x = load4<VEC_A>(a.act, m0 + row, k0 + 4 * c4, a.rows, K);
+            if (!FORWARD) {  // (grad_out * scale) first, as the reference does
+                const int o = k0 + 4 * c4;
+                x.x = x.x * (o + 0 < K ? a.scale[o + 0] : 0.0f);
+                x.y = x.y * (o + 1 < K ? a.scale[o + 1] : 0.0f);
+                x.z = x.z * (o + 2 < K ? a.scale[o + 2] : 0.0f);
+                x.w = x.w * (o + 3 < K ? a.scale[o + 3] : 0.0f);
+            }
+            ra[p] = x;
+        }
+        if (FORWARD) {
+            // thread -> (output row n, group g of the slab): 4 consecutive k of one weight row
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int idx = tid + kGemmThreads * p;
+                const int o = n0 + (idx >> 3), g = (k0 >> 2) + (idx & 7);
+                rw[p] = fetch_group(a.state, (size_t)o * gpr + g, last_group, o < a.out_features && g < gpr);
+            }
+        } else {
+            // thread -> (4 consecutive weight rows o = k, group g of the tile's columns)
+            const int oq = tid & 7, g = (n0 >> 2) + (tid >> 3);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int o = k0 + 4 * oq + r;
+                rw[r] = fetch_group(a.state, (size_t)o * gpr + g, last_group, o < a.out_features && g < gpr);
+            }
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int idx = tid + kGemmThreads * p;
+            const int row = idx >> 3, c4 = idx & 7;
+            store_split(lds_a, tile_offset(row, c4 >> 1, c4 & 1), ra[p].x, ra[p].y, ra[p].z, ra[p].w);
+        }
+        if (FORWARD) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int idx = tid + kGemmThreads * p;
+                const int n = idx >> 3, g = idx & 7;
+                const uint32_t lo = pack_bf16(ternary_of(rw[p], 0, a.cd), ternary_of(rw[p], 1, a.cd));
+                const uint32_t hi = pack_bf16(ternary_of(rw[p], 2, a.cd), ternary_of(rw[p], 3, a.cd));
+                *reinterpret_cast<uint2*>(lds_b + tile_offset(n, g >> 1, g & 1)) = make_uint2(lo, hi);
+            }
+        } else {
+            const int oq = tid & 7, g = tid >> 3;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {  // column n = 4 g + j of the tile, k = 4 oq .. 4 oq + 3
+                const uint32_t lo = pack_bf16(ternary_of(rw[0], j, a.cd), ternary_of(rw[1], j, a.cd));
+                const uint32_t hi = pack_bf16(ternary_of(rw[2], j, a.cd), ternary_of(rw[3], j, a.cd));
+                *reinterpret_cast<uint2*>(lds_b + tile_offset(4 * g + j, oq >> 1, oq & 1)) = make_uint2(lo, hi);
+            }
+        }
+    };
+
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += kK) {
+        stage();
+        __syncthreads();
+        if (k0 + kK < K) fetch(k0 + kK);
+#pragma unroll
+        for (int s = 0; s < kK / 16; ++s) {
+            const int chunk = 2 * s + kh;  // lane half kh holds k = 8 chunk .. 8 chunk + 7
+            bf16x8 fb[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb[j] = read_operand(lds_b, wn0 + 32 * j + l32, chunk);
+#pragma unroll
+            for (int plane = 0; plane < 3; ++plane) {
+                bf16x8 fa[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) fa[i] = read_operand(lds_a + plane * kPlaneBytes, wm0 + 32 * i + l32, chunk);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wn0 + 32 * j + l32;
+            const float s = (FORWARD && col < N) ? a.scale[col] : 1.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm0 + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+                if (row < a.rows && col < N) a.c[(size_t)row * N + col] = FORWARD ? acc[i][j][r] * s : acc[i][j][r];
+            }
+        }
+}
+
+template <bool FORWARD>
+hipError_t launch_lin3(hipStream_t stream, const float* act, const uint8_t* state, const float* scale, float* c,
+                       int C, int rows, int in_features, int out_features) {
+    Lin3Args a;
+    a.act = act;
+    a.state = state;
+    a.scale = scale;
+    a.c = c;
+    a.cd = make_codec(C);
+    a.rows = rows;
+    a.in_features = in_features;
+    a.out_features = out_features;
+    const int N = FORWARD ? out_features : in_features;
+    const int K = FORWARD ? in_features : out_features;
+    const dim3 grid((N + kT - 1) / kT, (rows + kT - 1) / kT);
+    const bool vec_a = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(act) & 15u) == 0);
+    const bool whole = rows % kT == 0 && N % kT == 0 && K % kK == 0 && vec_a &&
+                       (reinterpret_cast<uintptr_t>(scale) & 15u) == 0 &&
+                       (uint64_t)rows * (uint64_t)K * 4u < (1ull << 32) &&
+                       (uint64_t)out_features * (uint64_t)in_features * 3u / 4u < (1ull << 32);
+    if (whole)
+        hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD>), grid, dim3(kGemmThreads), 0, stream, a);
+    else if (vec_a)
+        hipLaunchKernelGGL((counter_linear_bf16x3_edge_kernel<FORWARD, true>), grid, dim3(kGemmThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((counter_linear_bf16x3_edge_kernel<FORWARD, false>), grid, dim3(kGemmThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_forward(hipStream_t stream, const float* x, const uint8_t* state, const float* scale, float* y,
+                          int C, int batch, int in_features, int out_features) {
+    return launch_lin3<true>(stream, x, state, scale, y, C, batch, in_features, out_features);
+}
+
+hipError_t launch_backward_input(hipStream_t stream, const float* grad_out, const uint8_t* state,
+                                 const float* scale, float* grad_x, int C, int batch, int in_features,
+                                 int out_features) {
+    return launch_lin3<false>(stream, grad_out, state, scale, grad_x, C, batch, in_features, out_features);
+}
+
+}  // namespace mcc
