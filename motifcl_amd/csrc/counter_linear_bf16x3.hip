@@ -18,10 +18,14 @@
 // line multiplies by the scale first, as kernels/compact_counter.cl:262-267 does).  Non-finite
 // activations are outside this kernel's contract (inf - inf in the split).
 //
-// Tile: 128 x 128 per workgroup of 4 waves (2 x 2, 64 x 64 each), 32-deep slabs.  LDS holds the
-// three activation planes and the weight tile as [row][32 bf16] = 64-byte rows whose four
-// 16-byte chunks are XOR-swizzled with bits 1-2 of the row, which makes the 16-byte MFMA operand
-// reads (lane = row, 8 consecutive k) conflict-free without padding: 32 KiB per workgroup.
+// Tile: 128 rows x 128 or 256 columns per workgroup of 4 or 8 waves (64 x 64 each), 32-deep
+// slabs.  LDS holds the three activation planes and the weight tile as [row][32 bf16] = 64-byte
+// rows whose four 16-byte chunks are XOR-swizzled with bits 1-2 of the row, which makes the
+// 16-byte MFMA operand reads (lane = row, 8 consecutive k) conflict-free without padding:
+// 32 or 40 KiB per workgroup.  Splitting and decoding are done by the thread that fetched the
+// data, on its way into LDS; per slab and thread that is about 200 VALU instructions against
+// 24 MFMAs, so the kernel runs near a third of the bf16 matrix peak -- twice the fp32 matrix
+// peak in algorithmic flops.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -97,15 +101,20 @@ __device__ __forceinline__ bf16x8 read_operand(const uint8_t* tile, int row, int
 // Whole tiles and whole slabs (rows, N multiples of 128, K a multiple of 32, 16-byte aligned
 // activation and scale, buffers below 4 GiB): nothing is checked, every address is a per-thread
 // 32-bit offset computed once plus a per-slab constant.
-template <bool FORWARD>
-__global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_kernel(Lin3Args a) {
+// WN waves side by side (each 64 columns) times 2 waves down: the tile is 128 rows x 64 WN columns
+// and the split of an activation slab is shared by that many columns.
+template <bool FORWARD, int WN>
+__global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16x3_kernel(Lin3Args a) {
+    constexpr int kThreads = 128 * WN;
+    constexpr int kTN = 64 * WN;
+    constexpr int kA4 = kT * kK / 4 / kThreads;  // float4 of activation per thread and slab
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * kPlaneBytes];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[kPlaneBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[kTN * kRowBytes];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, kh = lane >> 5;
-    const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
-    const int m0 = blockIdx.y * kT, n0 = blockIdx.x * kT;
+    const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
+    const int m0 = blockIdx.y * kT, n0 = blockIdx.x * kTN;
     const int K = FORWARD ? a.in_features : a.out_features;
     const int N = FORWARD ? a.out_features : a.in_features;
     const uint32_t gpr = (uint32_t)a.in_features >> 2;
@@ -119,19 +128,23 @@ __global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_kernel(
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    // thread (row = tid / 8 + 32 p, c4 = tid % 8) stages 4 activations per p; byte offsets
+    // thread (row = tid / 8 + (threads / 8) p, c4 = tid % 8) stages 4 activations per p; byte offsets
     const int c4 = tid & 7, row0 = tid >> 3;
-    uint32_t off_a[4], off_w[4];
-    int lds_off_a[4], lds_off_b[4];
+    uint32_t off_a[kA4], off_w[4];
+    int lds_off_a[kA4], lds_off_b[4];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int row = row0 + 32 * p;
+    for (int p = 0; p < kA4; ++p) {
+        const int row = row0 + (kThreads / 8) * p;
         off_a[p] = ((uint32_t)(m0 + row) * (uint32_t)K + 4u * c4) * 4u;
         lds_off_a[p] = tile_offset(row, c4 >> 1, c4 & 1);
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
         if (FORWARD) {
-            // (weight row n = row, group c4 of the slab)
-            off_w[p] = 3u * ((uint32_t)(n0 + row) * gpr + (uint32_t)c4);
-            lds_off_b[p] = lds_off_a[p];
+            // (weight row n = tid / 8 + (threads / 8) p, group c4 of the slab)
+            const int n = row0 + (kThreads / 8) * p;
+            off_w[p] = 3u * ((uint32_t)(n0 + n) * gpr + (uint32_t)c4);
+            lds_off_b[p] = tile_offset(n, c4 >> 1, c4 & 1);
         } else {
             // (weight rows k = 4 oq + p with oq = tid % 8, group g = tid / 8 of the tile's columns)
             off_w[p] = 3u * ((uint32_t)(4 * c4 + p) * gpr + (uint32_t)(n0 >> 2) + (uint32_t)row0);
@@ -140,17 +153,20 @@ __global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_kernel(
     }
     const uint32_t w_step = FORWARD ? 3u * (kK / 4) : 3u * kK * gpr;  // packed bytes per slab
 
-    float4 ra[4];
+    float4 ra[kA4];
     uint32_t rw[4];
     auto fetch = [&](int k0, uint32_t w_base) {
         float4 sc = make_float4(1.f, 1.f, 1.f, 1.f);
         if (!FORWARD) sc = *reinterpret_cast<const float4*>(a.scale + k0 + 4 * c4);
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
+        for (int p = 0; p < kA4; ++p) {
             const float4 x = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.act) + off_a[p] +
                                                               4u * (uint32_t)k0);
             // (grad_out * scale) first, as the reference does
             ra[p] = FORWARD ? x : make_float4(x.x * sc.x, x.y * sc.y, x.z * sc.z, x.w * sc.w);
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
             // one 4-byte load per packed group; the tensor's last group has no byte after it and
             // is fetched one byte early
             const uint32_t off = off_w[p] + w_base;
@@ -163,7 +179,7 @@ __global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_kernel(
     auto ternary = [&](uint32_t word, int k) { return (float)(code_q(code_of(word, k), a.cd) - 1); };
     auto stage = [&]() {
 #pragma unroll
-        for (int p = 0; p < 4; ++p) store_split(lds_a, lds_off_a[p], ra[p].x, ra[p].y, ra[p].z, ra[p].w);
+        for (int p = 0; p < kA4; ++p) store_split(lds_a, lds_off_a[p], ra[p].x, ra[p].y, ra[p].z, ra[p].w);
         if (FORWARD) {
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
@@ -369,14 +385,21 @@ hipError_t launch_lin3(hipStream_t stream, const float* act, const uint8_t* stat
     a.out_features = out_features;
     const int N = FORWARD ? out_features : in_features;
     const int K = FORWARD ? in_features : out_features;
-    const dim3 grid((N + kT - 1) / kT, (rows + kT - 1) / kT);
     const bool vec_a = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(act) & 15u) == 0);
     const bool whole = rows % kT == 0 && N % kT == 0 && K % kK == 0 && vec_a &&
                        (reinterpret_cast<uintptr_t>(scale) & 15u) == 0 &&
                        (uint64_t)rows * (uint64_t)K * 4u < (1ull << 32) &&
                        (uint64_t)out_features * (uint64_t)in_features * 3u / 4u < (1ull << 32);
+    // 256-column tiles (8 waves) share one split of the activation slab between twice as many
+    // columns: +15 % when there are enough of them to fill the device
+    if (whole && N % 256 == 0 && (long)(rows / kT) * (N / 256) >= 256) {
+        hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 4>), dim3(N / 256, rows / kT), dim3(512), 0, stream,
+                           a);
+        return hipGetLastError();
+    }
+    const dim3 grid((N + kT - 1) / kT, (rows + kT - 1) / kT);
     if (whole)
-        hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD>), grid, dim3(kGemmThreads), 0, stream, a);
+        hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 2>), grid, dim3(kGemmThreads), 0, stream, a);
     else if (vec_a)
         hipLaunchKernelGGL((counter_linear_bf16x3_edge_kernel<FORWARD, true>), grid, dim3(kGemmThreads), 0, stream, a);
     else

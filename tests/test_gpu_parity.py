@@ -258,7 +258,8 @@ def test_two_identical_fused_updates_agree_exactly(ops, oracle):
 # multiple of 4), both tile sizes, and a full-range state (codes the update cannot produce)
 LINEAR_SHAPES = [(2, 4, 2, 3), (37, 68, 35, 3), (64, 256, 256, 11), (100, 288, 768, 11),
                  (130, 768, 290, 11), (2048, 1024, 1280, 11), (1500, 2048, 1027, 4), (1, 4, 1, 11),
-                 (128, 128, 128, 11), (256, 384, 256, 3), (128, 4096, 128, 11), (384, 160, 2048, 1)]
+                 (128, 128, 128, 11), (256, 384, 256, 3), (128, 4096, 128, 11), (384, 160, 2048, 1),
+                 (4096, 256, 2048, 11), (4096, 2048, 256, 11)]  # 256-column tiles: forward, grad_x
 
 
 @pytest.mark.parametrize("shape", LINEAR_SHAPES, ids=lambda s: "N%d_in%d_out%d_C%d" % s)
