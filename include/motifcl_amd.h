@@ -155,6 +155,26 @@ int mcc_compact_counter_apply_update_fused(
     float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
 
 /*
+ * How the weight-gradient contraction (inside the two-kernel fused step and in
+ * mcc_matmul_transpose_a_f32) multiplies.  Process-wide; no counterpart in the
+ * reference.
+ *   MCC_CONTRACTION_FP32    the fp32 matrix instruction (default)
+ *   MCC_CONTRACTION_BF16X6  both operands split into three bf16 terms, six bf16
+ *                           matrix passes per product: per-product error of one
+ *                           binary32 rounding, as the fp32 instruction, at about
+ *                           1.7 x its speed.  Used for whole 128 x 128 tiles and
+ *                           token counts that are multiples of 32; other shapes
+ *                           silently use the fp32 instruction.  The two modes give
+ *                           gradients that differ in the last bits, so counters
+ *                           whose tick lands within that distance of a rounding
+ *                           boundary may come out differently.
+ */
+#define MCC_CONTRACTION_FP32 0
+#define MCC_CONTRACTION_BF16X6 1
+int mcc_set_contraction_mode(int mode);
+int mcc_get_contraction_mode(void);
+
+/*
  * c[m,n] = a[k,m]^T . b[k,n], fp32, row-major.
  * Replaces matmul_transpose_a (include/motifcl/ops/matmul.hpp:8,
  * src/ops/matmul.cpp:1416-1418), the producer of the dense weight gradient

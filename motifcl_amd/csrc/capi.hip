@@ -38,6 +38,10 @@ constexpr size_t kIntMax = static_cast<size_t>(std::numeric_limits<int>::max());
 constexpr unsigned kDefaultStripSpinLimit = 1u << 24;
 std::atomic<unsigned> g_strip_spin_limit{kDefaultStripSpinLimit};
 
+// 0: weight-gradient contraction on the fp32 matrix instruction; 1: split-bf16 form where the
+// shape allows it
+std::atomic<int> g_contraction_mode{0};
+
 // Shared shape/codec checks.  `what` names the operation in messages.
 bool check_codec(const char* what, size_t C, size_t in_features, size_t out_features) {
     if (in_features == 0 || out_features == 0) {
@@ -321,7 +325,8 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
         // the chunk slices start at grad_w: the chunk sums are reduced in place into slice 0
-        e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features, grad_w);
+        e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features, grad_w,
+                                    g_contraction_mode.load());
     }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
     {
@@ -332,6 +337,15 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update launch failed");
     return MCC_OK;
 }
+
+int mcc_set_contraction_mode(int mode) {
+    if (mode != MCC_CONTRACTION_FP32 && mode != MCC_CONTRACTION_BF16X6)
+        return fail(MCC_E_INVALID, "unknown contraction mode");
+    g_contraction_mode.store(mode);
+    return MCC_OK;
+}
+
+int mcc_get_contraction_mode(void) { return g_contraction_mode.load(); }
 
 int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, const float* b,
                                size_t b_nbytes, float* c, size_t c_nbytes, size_t k, size_t m,
@@ -360,7 +374,7 @@ int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, co
     hipError_t e;
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
-        e = mcc::launch_gemm_tn_f32(s, a, b, c, (int)k, (int)m, (int)n, temp);
+        e = mcc::launch_gemm_tn_f32(s, a, b, c, (int)k, (int)m, (int)n, temp, g_contraction_mode.load());
     }
     if (temp) {
         const hipError_t ef = hipFreeAsync(temp, s);

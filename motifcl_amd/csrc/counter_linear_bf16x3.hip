@@ -30,20 +30,13 @@
 
 #include <cstdint>
 
+#include "bf16_split.hpp"
 #include "counter_math.hpp"
 #include "gemm_tile.hpp"
 #include "launch.hpp"
 
 namespace mcc {
 namespace {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-
-constexpr int kT = 128;        // tile rows and columns
-constexpr int kK = 32;         // slab depth
-constexpr int kRowBytes = 64;  // 32 bf16
-constexpr int kPlaneBytes = kT * kRowBytes;
 
 struct Lin3Args {
     const float* act;      // [rows, K]
@@ -53,30 +46,6 @@ struct Lin3Args {
     Codec cd;
     int rows, in_features, out_features;
 };
-
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    const bf16x2 p = {(__bf16)a, (__bf16)b};  // round to nearest even
-    return __builtin_bit_cast(uint32_t, p);
-}
-__device__ __forceinline__ float bf16_lo(uint32_t p) { return __uint_as_float(p << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
-
-// Byte offset of 8-byte piece `half` of 16-byte chunk `chunk` of row `row` in a swizzled tile.
-__device__ __forceinline__ int tile_offset(int row, int chunk, int half) {
-    return row * kRowBytes + ((chunk ^ ((row >> 1) & 3)) << 4) + (half << 3);
-}
-
-// Splits four activations into their three bf16 planes and stores each as 8 bytes.
-__device__ __forceinline__ void store_split(uint8_t* planes, int offset, float x0, float x1, float x2, float x3) {
-    const uint32_t h01 = pack_bf16(x0, x1), h23 = pack_bf16(x2, x3);
-    const float r0 = x0 - bf16_lo(h01), r1 = x1 - bf16_hi(h01), r2 = x2 - bf16_lo(h23), r3 = x3 - bf16_hi(h23);
-    const uint32_t m01 = pack_bf16(r0, r1), m23 = pack_bf16(r2, r3);
-    const float s0 = r0 - bf16_lo(m01), s1 = r1 - bf16_hi(m01), s2 = r2 - bf16_lo(m23), s3 = r3 - bf16_hi(m23);
-    const uint32_t l01 = pack_bf16(s0, s1), l23 = pack_bf16(s2, s3);
-    *reinterpret_cast<uint2*>(planes + offset) = make_uint2(h01, h23);
-    *reinterpret_cast<uint2*>(planes + kPlaneBytes + offset) = make_uint2(m01, m23);
-    *reinterpret_cast<uint2*>(planes + 2 * kPlaneBytes + offset) = make_uint2(l01, l23);
-}
 
 __device__ __forceinline__ uint32_t fetch_group(const uint8_t* state, size_t group, size_t last_group, bool valid) {
     if (!valid) return 0xffffffffu;  // marks "no weight": decoded to zero below
@@ -91,11 +60,6 @@ __device__ __forceinline__ uint32_t fetch_group(const uint8_t* state, size_t gro
 __device__ __forceinline__ float ternary_of(uint32_t word, int k, const Codec& cd) {
     const float t = (float)(code_q(code_of(word, k), cd) - 1);
     return word == 0xffffffffu ? 0.0f : t;
-}
-
-__device__ __forceinline__ bf16x8 read_operand(const uint8_t* tile, int row, int chunk) {
-    const uint4 v = *reinterpret_cast<const uint4*>(tile + tile_offset(row, chunk, 0));
-    return __builtin_bit_cast(bf16x8, v);
 }
 
 // Whole tiles and whole slabs (rows, N multiples of 128, K a multiple of 32, 16-byte aligned

@@ -109,11 +109,15 @@ size_t gemm_tn_slices(int k, int m, int n) { return (size_t)plan_gemm_tn(k, m, n
 // `slices` holds plan.splits * m * n floats when the plan splits the tokens (it may start at c);
 // it is not touched otherwise.
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n,
-                              float* slices) {
+                              float* slices, int mode) {
     const GemmTnPlan plan = plan_gemm_tn(k, m, n);
     float* out = plan.splits > 1 ? slices : c;
     if (plan.splits > 1 && !slices) return hipErrorInvalidValue;
-    hipError_t e = plan.tile == 128 ? launch_tile<128, 128>(stream, a, b, out, k, m, n, plan)
+    hipError_t e;
+    if (mode == 1 && gemm_tn_bf16x6_supports(a, b, k, m, n, plan))
+        e = launch_gemm_tn_bf16x6(stream, a, b, out, k, m, n, plan);
+    else
+        e = plan.tile == 128 ? launch_tile<128, 128>(stream, a, b, out, k, m, n, plan)
                                     : launch_tile<64, 64>(stream, a, b, out, k, m, n, plan);
     if (e != hipSuccess || plan.splits == 1) return e;
     const size_t mn = (size_t)m * n;

@@ -40,8 +40,13 @@ struct GemmTnPlan {
 };
 GemmTnPlan plan_gemm_tn(int k, int m, int n);
 size_t gemm_tn_slices(int k, int m, int n);
+// mode: 0 = fp32 matrix instruction; 1 = both operands split into three bf16 terms, six bf16
+// passes (gemm_tn_bf16x6.hip), where the shape allows it
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c,
-                              int k, int m, int n, float* slices);
+                              int k, int m, int n, float* slices, int mode = 0);
+bool gemm_tn_bf16x6_supports(const float* a, const float* b, int k, int m, int n, const GemmTnPlan& plan);
+hipError_t launch_gemm_tn_bf16x6(hipStream_t stream, const float* a, const float* b, float* out,
+                                 int k, int m, int n, const GemmTnPlan& plan);
 
 // Fused step that keeps G in the contraction's accumulators (counter_fused_strip.hip).
 // Shapes: in_features and out_features multiples of 128; lr_scale == 0 is implied.

@@ -22,6 +22,8 @@ SIGNATURES = {
     "mcc_compact_counter_apply_update_fused": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
                        _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
+    "mcc_set_contraction_mode": (ctypes.c_int, [ctypes.c_int]),
+    "mcc_get_contraction_mode": (ctypes.c_int, []),
     "mcc_matmul_transpose_a_f32": (ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz]),
     "mcc_compact_counter_decode_weight": (ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz]),
     "mcc_compact_counter_forward_u8": (

@@ -153,3 +153,15 @@ def adam_update(param, grad, m, v, lr, beta1, beta2, eps, step, weight_decay=0.0
     _lib.check(L.mcc_adam_update_f32(_stream(), *_buf(param, torch.float32), *_buf(grad, torch.float32),
                                      *_buf(m, torch.float32), *_buf(v, torch.float32), param.numel(),
                                      lr, beta1, beta2, eps, step, weight_decay))
+
+
+CONTRACTION_FP32, CONTRACTION_BF16X6 = 0, 1
+
+
+def set_contraction_mode(mode):
+    """Process-wide choice of the weight-gradient contraction: fp32 matrix instruction or split bf16."""
+    _lib.check(_lib.load().mcc_set_contraction_mode(int(mode)))
+
+
+def get_contraction_mode():
+    return int(_lib.load().mcc_get_contraction_mode())
