@@ -34,6 +34,17 @@ __device__ __forceinline__ int tile_offset(int row, int chunk, int half) {
     return row * kRowBytes + ((chunk ^ ((row >> 1) & 3)) << 4) + (half << 3);
 }
 
+// The same for a stager that transposes: its wave writes, in one instruction, 8-byte pieces of
+// rows r, r + 4, ..., r + 28.  In the layout above those rows are 256 bytes -- one sweep of the
+// banks -- apart and the write is an 8-way bank conflict.  Here row r sits at position
+// (r % 4) * 32 + r / 4, so the eight rows are 512 contiguous bytes; the chunk swizzle (r % 4, and
+// bit 4 of r so that rows 16 apart differ) keeps both those writes and the operand reads
+// (consecutive rows, one chunk) conflict-free.
+__device__ __forceinline__ int dealt_tile_offset(int row, int chunk, int half) {
+    const int swizzle = (row & 3) ^ ((row >> 3) & 2);
+    return (((row & 3) * (kT / 4)) + (row >> 2)) * kRowBytes + ((chunk ^ swizzle) << 4) + (half << 3);
+}
+
 // Splits four activations into their three bf16 planes and stores each as 8 bytes.
 __device__ __forceinline__ void store_split(uint8_t* planes, int offset, float x0, float x1, float x2, float x3) {
     const uint32_t h01 = pack_bf16(x0, x1), h23 = pack_bf16(x2, x3);
@@ -48,6 +59,10 @@ __device__ __forceinline__ void store_split(uint8_t* planes, int offset, float x
 
 __device__ __forceinline__ bf16x8 read_operand(const uint8_t* tile, int row, int chunk) {
     const uint4 v = *reinterpret_cast<const uint4*>(tile + tile_offset(row, chunk, 0));
+    return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ bf16x8 read_dealt_operand(const uint8_t* tile, int row, int chunk) {
+    const uint4 v = *reinterpret_cast<const uint4*>(tile + dealt_tile_offset(row, chunk, 0));
     return __builtin_bit_cast(bf16x8, v);
 }
 

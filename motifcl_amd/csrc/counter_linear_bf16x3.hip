@@ -78,7 +78,9 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, kh = lane >> 5;
     const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
-    const int m0 = blockIdx.y * kT, n0 = blockIdx.x * kTN;
+    // the activation panel weighs 4 bytes an element, the packed weight panel 0.75: flat bands
+    const TileXY tile = xcd_tile(gridDim.x, gridDim.y, 4);
+    const int m0 = tile.y * kT, n0 = tile.x * kTN;
     const int K = FORWARD ? a.in_features : a.out_features;
     const int N = FORWARD ? a.out_features : a.in_features;
     const uint32_t gpr = (uint32_t)a.in_features >> 2;

@@ -69,6 +69,32 @@ __device__ __forceinline__ TilePos tile_pos() {
     return p;
 }
 
+// Which tile of a tiles_x x tiles_y grid the calling workgroup computes.  Workgroups are dealt to
+// the 8 XCDs round-robin by linear id, and each XCD has an L2 of its own: a tile order that
+// follows the launch order puts neighbouring tiles -- which share operand panels -- on eight
+// different L2s.  Here workgroups w, w + 8, w + 16, ... (one XCD) take consecutive tiles of an
+// order that walks bands of `band_rows` tile rows column by column, so the workgroups resident
+// together on an XCD cover a compact block of tiles and fetch each panel slab once between them.
+// A bijection for any grid; gridDim.x * gridDim.y must equal tiles_x * tiles_y.
+struct TileXY {
+    int x, y;
+};
+__device__ __forceinline__ TileXY xcd_tile(int tiles_x, int tiles_y, int band_rows) {
+    const uint32_t total = (uint32_t)tiles_x * (uint32_t)tiles_y;
+    const uint32_t w = blockIdx.x + blockIdx.y * gridDim.x;
+    const uint32_t xcd = w & 7u, local = w >> 3;
+    const uint32_t base = total >> 3, rem = total & 7u;
+    const uint32_t t = xcd * base + (xcd < rem ? xcd : rem) + local;
+    const uint32_t band_tiles = (uint32_t)band_rows * (uint32_t)tiles_x;
+    const uint32_t band = t / band_tiles, within = t - band * band_tiles;
+    const uint32_t left = (uint32_t)tiles_y - band * (uint32_t)band_rows;
+    const uint32_t rows = left < (uint32_t)band_rows ? left : (uint32_t)band_rows;
+    TileXY r;
+    r.x = (int)(within / rows);
+    r.y = (int)(band * (uint32_t)band_rows + within % rows);
+    return r;
+}
+
 // Accumulates the BM x BN tile at (m0, n0) over all K tokens into acc (zeroed here).  lds holds
 // TileCfg::kLdsFloats floats.  Ends with a barrier, so lds may be reused right after.
 // Accumulator layout (v_mfma_f32_32x32x2_f32): acc[i][j][r] is row

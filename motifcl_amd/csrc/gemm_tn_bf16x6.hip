@@ -31,7 +31,8 @@ __global__ __launch_bounds__(kGemmThreads, 3) void gemm_tn_bf16x6_kernel(const f
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, kh = lane >> 5;
     const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
-    const int m0 = blockIdx.y * kT, n0 = blockIdx.x * kT;
+    const TileXY tile = xcd_tile(gridDim.x, gridDim.y, 8);
+    const int m0 = tile.y * kT, n0 = tile.x * kT;
     const int k_begin = blockIdx.z * chunk_tokens;
     const int k_len = K - k_begin < chunk_tokens ? K - k_begin : chunk_tokens;
     c += (size_t)blockIdx.z * M * N;
@@ -44,13 +45,15 @@ __global__ __launch_bounds__(kGemmThreads, 3) void gemm_tn_bf16x6_kernel(const f
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    // thread (kq = tid % 8, cq = tid / 8): tokens 4 kq .. 4 kq + 3 of the slab, columns 4 cq .. 4 cq + 3
-    const int kq = tid & 7, cq = tid >> 3;
+    // thread (kq, cq): tokens 4 kq .. 4 kq + 3 of the slab, columns 4 cq .. 4 cq + 3.  Eight
+    // neighbouring lanes take neighbouring cq, so that a wave's load is eight whole 128-byte lines
+    // (lanes that alternate between rows are fetched one 16-byte request at a time).
+    const int kq = lane >> 3, cq = 8 * wave + (lane & 7);
     const uint32_t off_a = ((uint32_t)(k_begin + 4 * kq) * (uint32_t)M + (uint32_t)(m0 + 4 * cq)) * 4u;
     const uint32_t off_b = ((uint32_t)(k_begin + 4 * kq) * (uint32_t)N + (uint32_t)(n0 + 4 * cq)) * 4u;
     int lds_off[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) lds_off[j] = tile_offset(4 * cq + j, kq >> 1, kq & 1);
+    for (int j = 0; j < 4; ++j) lds_off[j] = dealt_tile_offset(4 * cq + j, kq >> 1, kq & 1);
 
     float4 ra[4], rb[4];
     auto fetch = [&](int k0) {
@@ -87,8 +90,8 @@ __global__ __launch_bounds__(kGemmThreads, 3) void gemm_tn_bf16x6_kernel(const f
             for (int p = 0; p < 3; ++p)
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    fa[p][i] = read_operand(lds_a + p * kPlaneBytes, wm0 + 32 * i + l32, chunk);
-                    fb[p][i] = read_operand(lds_b + p * kPlaneBytes, wn0 + 32 * i + l32, chunk);
+                    fa[p][i] = read_dealt_operand(lds_a + p * kPlaneBytes, wm0 + 32 * i + l32, chunk);
+                    fb[p][i] = read_dealt_operand(lds_b + p * kPlaneBytes, wn0 + 32 * i + l32, chunk);
                 }
             // smallest terms first
             constexpr int pa[6] = {1, 0, 2, 0, 1, 0};

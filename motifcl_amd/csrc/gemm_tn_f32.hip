@@ -21,8 +21,9 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tn_kernel(const float* __re
     using Cfg = TileCfg<BM, BN>;
     __shared__ float lds[DIRECT ? DirectCfg<BM, BN>::kLdsFloats : Cfg::kLdsFloats];
     const TilePos tp = tile_pos<BM, BN>();
-    const int m0 = blockIdx.y * BM;
-    const int n0 = blockIdx.x * BN;
+    const TileXY tile = xcd_tile(gridDim.x, gridDim.y, 8);
+    const int m0 = tile.y * BM;
+    const int n0 = tile.x * BN;
     const int k_begin = blockIdx.z * chunk;
     const int k_len = K - k_begin < chunk ? K - k_begin : chunk;
     a += (size_t)k_begin * M;
