@@ -277,6 +277,19 @@ void mcc_profiler_enable(int on);
 void mcc_profiler_reset(void);
 int mcc_profiler_query(const char* kernel_name, double* total_ms, uint64_t* launches);
 
+/*
+ * Shader-clock probe (a measurement aid with no counterpart in the reference).
+ * Enqueues a one-wave kernel on `stream` that sleeps for `seconds` (at most 2) of
+ * the constant-rate wall clock and writes two 64-bit counts to the device buffer
+ * `out`: out[0] wall-clock ticks, out[1] shader cycles over the same stretch.
+ * Launched on a side stream while other kernels run it gives the frequency they
+ * ran at: MHz = out[1] / out[0] * wall_clock_khz / 1000.  Matrix-core peaks are
+ * quoted at the maximum engine clock; under load the power limit holds the clock
+ * below it.
+ */
+int mcc_clock_probe(void* stream, uint64_t* out, size_t out_nbytes, double seconds);
+int mcc_wall_clock_khz(int* khz);
+
 #ifdef __cplusplus
 }
 #endif

@@ -4,8 +4,10 @@
 // Each subtraction is exact (24 significant bits are peeled off 8 at a time; only numbers within
 // 2^16 of the smallest normal lose their tail), and a bf16 x bf16 product is exact in binary32.
 // Operand tiles live in LDS as [row][32 bf16] = 64-byte rows whose four 16-byte chunks are
-// XOR-swizzled with bits 1-2 of the row, which makes the 16-byte MFMA operand reads (lane = row,
-// 8 consecutive k) conflict-free without padding.
+// XOR-swizzled with bits 2-3 of the row.  A 16-byte operand read (lane = row, 8 consecutive k) is
+// served 16 lanes a cycle, all 64 banks at once: rows r, r + 4, r + 8, r + 12 start in the same
+// banks and the swizzle sends them to four different chunks, so the read is conflict-free
+// without padding (measured: SQ_LDS_BANK_CONFLICT drops from half of the LDS cycles to none).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -31,7 +33,7 @@ __device__ __forceinline__ float bf16_hi(uint32_t p) { return __uint_as_float(p 
 
 // Byte offset of 8-byte piece `half` of 16-byte chunk `chunk` of row `row` in a swizzled tile.
 __device__ __forceinline__ int tile_offset(int row, int chunk, int half) {
-    return row * kRowBytes + ((chunk ^ ((row >> 1) & 3)) << 4) + (half << 3);
+    return row * kRowBytes + ((chunk ^ ((row >> 2) & 3)) << 4) + (half << 3);
 }
 
 // The same for a stager that transposes: its wave writes, in one instruction, 8-byte pieces of

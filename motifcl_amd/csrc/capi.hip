@@ -600,6 +600,28 @@ int mcc_memset_zero(void* stream, void* dst, size_t nbytes) {
     return MCC_OK;
 }
 
+int mcc_wall_clock_khz(int* khz) {
+    if (!khz) return fail(MCC_E_INVALID, "wall_clock_khz received a null pointer");
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(khz, hipDeviceAttributeWallClockRate, dev);
+    if (e != hipSuccess) return hip_fail(e, "wall_clock_khz query failed");
+    return MCC_OK;
+}
+
+int mcc_clock_probe(void* stream, uint64_t* out, size_t out_nbytes, double seconds) {
+    if (!out || out_nbytes < 2 * sizeof(uint64_t)) return fail(MCC_E_INVALID, "clock_probe needs a 16-byte device buffer");
+    if (!(seconds > 0.0) || seconds > 2.0) return fail(MCC_E_INVALID, "clock_probe duration must be in (0, 2] seconds");
+    int khz = 0;
+    const int rc = mcc_wall_clock_khz(&khz);
+    if (rc != MCC_OK) return rc;
+    const unsigned long long ticks = (unsigned long long)(seconds * 1e3 * (double)khz);
+    const hipError_t e =
+        mcc::launch_clock_probe(static_cast<hipStream_t>(stream), reinterpret_cast<unsigned long long*>(out), ticks);
+    if (e != hipSuccess) return hip_fail(e, "clock_probe launch failed");
+    return MCC_OK;
+}
+
 void mcc_profiler_enable(int on) {
     Profiler& p = profiler();
     std::lock_guard<std::mutex> lock(p.mu);

@@ -20,7 +20,7 @@
 //
 // Tile: 128 rows x 128 or 256 columns per workgroup of 4 or 8 waves (64 x 64 each), 32-deep
 // slabs.  LDS holds the three activation planes and the weight tile as [row][32 bf16] = 64-byte
-// rows whose four 16-byte chunks are XOR-swizzled with bits 1-2 of the row, which makes the
+// rows whose four 16-byte chunks are XOR-swizzled with bits 2-3 of the row, which makes the
 // 16-byte MFMA operand reads (lane = row, 8 consecutive k) conflict-free without padding:
 // 32 or 40 KiB per workgroup.  Splitting and decoding are done by the thread that fetched the
 // data, on its way into LDS; per slab and thread that is about 200 VALU instructions against

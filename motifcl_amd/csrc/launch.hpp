@@ -76,4 +76,7 @@ hipError_t launch_adam_update(hipStream_t stream, float* param, const float* gra
                               size_t n, float lr, float beta1, float beta2, float eps, float inv_bias1,
                               float inv_bias2, float weight_decay);
 
+// out[0] = wall-clock ticks slept (>= wall_ticks), out[1] = shader cycles over the same stretch
+hipError_t launch_clock_probe(hipStream_t stream, unsigned long long* out, unsigned long long wall_ticks);
+
 }  // namespace mcc

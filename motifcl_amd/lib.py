@@ -43,6 +43,8 @@ SIGNATURES = {
     "mcc_memcpy_d2h": (ctypes.c_int, [_vp, _vp, _vp, _sz]),
     "mcc_memset_zero": (ctypes.c_int, [_vp, _vp, _sz]),
     "mcc_stream_synchronize": (ctypes.c_int, [_vp]),
+    "mcc_clock_probe": (ctypes.c_int, [_vp, _vp, _sz, ctypes.c_double]),
+    "mcc_wall_clock_khz": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int)]),
     "mcc_profiler_enable": (None, [ctypes.c_int]),
     "mcc_profiler_reset": (None, []),
     "mcc_profiler_query": (ctypes.c_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),

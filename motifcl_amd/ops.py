@@ -1,6 +1,8 @@
 """Thin Python front of the C ABI.  torch is used only as the owner of device
 memory and of the current HIP stream; every computation happens in
 libmotifcl_amd.so."""
+import ctypes
+
 import torch
 
 from . import lib as _lib
@@ -165,3 +167,32 @@ def set_contraction_mode(mode):
 
 def get_contraction_mode():
     return int(_lib.load().mcc_get_contraction_mode())
+
+
+class ClockProbe:
+    """Shader clock while other kernels run: a one-wave kernel on a side stream sleeps for
+    `seconds` of the constant-rate wall clock and counts shader cycles over the same stretch.
+
+        probe = ClockProbe(0.05)      # starts now, on its own stream
+        ... launch the kernels under test on the current stream ...
+        torch.cuda.synchronize()
+        mhz = probe.mhz()
+    """
+
+    def __init__(self, seconds):
+        L = _lib.load()
+        khz = ctypes.c_int(0)
+        _lib.check(L.mcc_wall_clock_khz(ctypes.byref(khz)))
+        self._khz = khz.value
+        self._out = torch.zeros(2, dtype=torch.int64, device="cuda")
+        self._stream = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        _lib.check(L.mcc_clock_probe(ctypes.c_void_p(self._stream.cuda_stream), ctypes.c_void_p(self._out.data_ptr()),
+                                     16, float(seconds)))
+
+    def mhz(self):
+        self._stream.synchronize()
+        wall, cycles = (int(v) for v in self._out.tolist())
+        if wall <= 0:
+            raise RuntimeError("clock probe has not run")
+        return cycles / wall * self._khz / 1000.0

@@ -319,3 +319,19 @@ def test_known_answer_vectors_on_gpu(ops, oracle):
     for r in range(2):
         for i in range(4):
             assert gx[r, i] == go[r, 0] * 0.5 * tern[i] + go[r, 1] * 2.0 * tern[4 + i]
+
+
+@pytest.mark.gpu
+def test_clock_probe_reports_a_plausible_shader_clock():
+    # a measurement aid: one wave sleeps 20 ms of wall clock on a side stream and counts shader cycles
+    import torch
+    from motifcl_amd import ops
+    probe = ops.ClockProbe(0.02)
+    x = torch.randn(4096, 4096, device="cuda")
+    for _ in range(10):
+        x = x @ x * 1e-3
+    torch.cuda.synchronize()
+    mhz = probe.mhz()
+    assert 100.0 < mhz < 3000.0, mhz
+    with pytest.raises(RuntimeError):
+        ops.ClockProbe(5.0)
