@@ -42,9 +42,11 @@ __device__ __forceinline__ int tile_offset(int row, int chunk, int half) {
 // (r % 4) * 32 + r / 4, so the eight rows are 512 contiguous bytes; the chunk swizzle (r % 4, and
 // bit 4 of r so that rows 16 apart differ) keeps both those writes and the operand reads
 // (consecutive rows, one chunk) conflict-free.
+template <int ROWS = kT>
 __device__ __forceinline__ int dealt_tile_offset(int row, int chunk, int half) {
+    static_assert(ROWS % 16 == 0, "a quarter of the tile must be whole bank sweeps");
     const int swizzle = (row & 3) ^ ((row >> 3) & 2);
-    return (((row & 3) * (kT / 4)) + (row >> 2)) * kRowBytes + ((chunk ^ swizzle) << 4) + (half << 3);
+    return (((row & 3) * (ROWS / 4)) + (row >> 2)) * kRowBytes + ((chunk ^ swizzle) << 4) + (half << 3);
 }
 
 // Splits four activations into their three bf16 planes and stores each as 8 bytes.
@@ -63,8 +65,9 @@ __device__ __forceinline__ bf16x8 read_operand(const uint8_t* tile, int row, int
     const uint4 v = *reinterpret_cast<const uint4*>(tile + tile_offset(row, chunk, 0));
     return __builtin_bit_cast(bf16x8, v);
 }
+template <int ROWS = kT>
 __device__ __forceinline__ bf16x8 read_dealt_operand(const uint8_t* tile, int row, int chunk) {
-    const uint4 v = *reinterpret_cast<const uint4*>(tile + dealt_tile_offset(row, chunk, 0));
+    const uint4 v = *reinterpret_cast<const uint4*>(tile + dealt_tile_offset<ROWS>(row, chunk, 0));
     return __builtin_bit_cast(bf16x8, v);
 }
 

@@ -114,7 +114,8 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
         } else {
             // (weight rows k = 4 oq + p with oq = tid % 8, group g = tid / 8 of the tile's columns)
             off_w[p] = 3u * ((uint32_t)(4 * c4 + p) * gpr + (uint32_t)(n0 >> 2) + (uint32_t)row0);
-            lds_off_b[p] = tile_offset(4 * row0 + p, c4 >> 1, c4 & 1);  // column n = 4 g + p, k = 4 oq ..
+            // column n = 4 g + p, k = 4 oq ..: a wave writes rows 4 apart, hence the dealt row order
+            lds_off_b[p] = dealt_tile_offset<kTN>(4 * row0 + p, c4 >> 1, c4 & 1);
         }
     }
     const uint32_t w_step = FORWARD ? 3u * (kK / 4) : 3u * kK * gpr;  // packed bytes per slab
@@ -181,7 +182,8 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
             const int chunk = 2 * s + kh;
             bf16x8 fb[2];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) fb[j] = read_operand(lds_b, read_b[j], chunk);
+            for (int j = 0; j < 2; ++j)
+                fb[j] = FORWARD ? read_operand(lds_b, read_b[j], chunk) : read_dealt_operand<kTN>(lds_b, read_b[j], chunk);
 #pragma unroll
             for (int plane = 0; plane < 3; ++plane) {
                 bf16x8 fa[2];
