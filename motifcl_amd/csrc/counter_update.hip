@@ -269,6 +269,70 @@ __device__ __forceinline__ void update_row_streamed(const BatchArgs& a, const Up
     apply_streamed(t, row, lane, rc.tc, luts);
 }
 
+// One row of any length, 16-byte aligned, not the last of its tensor, by one wave in two passes
+// over the row: statistics first, ticks second.  The second pass finds the row in L2 or in the
+// memory-side cache as long as the rows in flight fit there (5 waves per SIMD: 5120 rows, i.e.
+// 100-230 MB at 5120-11008 weights a row); what the two passes buy is a register footprint of
+// one chunk instead of one row, i.e. the occupancy of a short row at any length, and no
+// hand-off between waves.  A chunk is kChunk iterations whose loads are issued back to back
+// (8 measured best against 4, 6 and 11).
+constexpr int kChunk = 8;
+
+template <bool WITH_GS>
+__device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const UpdateTensor& t, int row,
+                                                    int lane, Luts& luts) {
+    const uint32_t gpr = (uint32_t)t.in_features >> 2;
+    const int iters = (int)((gpr + kWave - 1) / kWave);
+    const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
+    uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    RowAcc acc;
+    for (int c0 = 0; c0 < iters; c0 += kChunk) {
+        float4 q[kChunk];
+        uint32_t w[WITH_GS ? kChunk : 1];
+#pragma unroll
+        for (int j = 0; j < kChunk; ++j) {
+            const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j);
+            const uint32_t gc = gi < gpr ? gi : gpr - 1;
+            q[j] = g_row[gc];
+            if (WITH_GS) w[j] = load_group_dword(s_row + 3u * gc);
+        }
+#pragma unroll
+        for (int j = 0; j < kChunk; ++j) {
+            // groups past the end add +0.0 (squares) and -+0.0 (0 * t): the sums do not change
+            const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j) < gpr;
+            const float g[4] = {live ? q[j].x : 0.0f, live ? q[j].y : 0.0f, live ? q[j].z : 0.0f,
+                                live ? q[j].w : 0.0f};
+            accumulate<WITH_GS>(acc, g, WITH_GS ? w[j] : 0u, a.cd);
+        }
+    }
+    const RowCtx rc = finish_row<WITH_GS>(a, t, row, lane, acc, luts);
+    if (!rc.fast_div) {
+        apply_streamed(t, row, lane, rc.tc, luts);
+        return;
+    }
+    const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
+    for (int c0 = 0; c0 < iters; c0 += kChunk) {
+        float4 q[kChunk];
+        uint32_t w[kChunk];
+#pragma unroll
+        for (int j = 0; j < kChunk; ++j) {
+            const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j);
+            const uint32_t gc = gi < gpr ? gi : gpr - 1;
+            q[j] = g_row[gc];
+            w[j] = load_group_dword(s_row + 3u * gc);
+        }
+#pragma unroll
+        for (int j = 0; j < kChunk; ++j) {
+            if (c0 + j < iters) {  // wave-uniform
+                const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j);
+                const float g[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
+                const uint32_t nw = tick_group<true>(w[j], g, rc.tc, luts, row_elem + 4u * gi);
+                if (gi < gpr) store_group(s_row + 3u * gi, nw);
+            }
+        }
+    }
+}
+
 // Minimum waves per SIMD the compiler must leave room for: the tick arithmetic has long
 // dependent chains, so the row's registers are budgeted to keep 3-4 waves resident for short
 // rows and 2 for the longest.
@@ -299,6 +363,26 @@ __global__ __launch_bounds__(kThreads, min_waves(ITERS)) void update_rows_kernel
         // byte after it for the 4-byte state load
         if (ITERS > 0 && row != t.out_features - 1)
             update_row_resident<(ITERS > 0 ? ITERS : 1), WITH_GS>(a, t, row, lane, luts);
+        else
+            update_row_streamed<WITH_GS>(a, t, row, lane, luts);
+    }
+}
+
+template <bool WITH_GS>
+__global__ __launch_bounds__(kThreads, 4) void update_rows_long_kernel(BatchArgs a) {
+    __shared__ Luts luts;
+    build_luts(luts, a.cd, a.geom);
+    const int lane = threadIdx.x;
+    int ti = 0;
+    for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
+        const int grow = __builtin_amdgcn_readfirstlane(grow_v);
+        ti = __builtin_amdgcn_readfirstlane(ti);
+        while (grow >= a.t[ti].row_start + a.t[ti].out_features) ++ti;  // monotonic
+        ti = __builtin_amdgcn_readfirstlane(ti);
+        const UpdateTensor t = a.t[ti];
+        const int row = grow - t.row_start;
+        if (row != t.out_features - 1)
+            update_row_two_pass<WITH_GS>(a, t, row, lane, luts);
         else
             update_row_streamed<WITH_GS>(a, t, row, lane, luts);
     }
@@ -507,6 +591,23 @@ hipError_t launch_split_variant(hipStream_t stream, const BatchArgs& a) {
     return hipGetLastError();
 }
 
+template <bool WITH_GS>
+hipError_t launch_long_variant(hipStream_t stream, const BatchArgs& a) {
+    static int blocks_per_cu = [] {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_long_kernel<WITH_GS>, kThreads, 0) != hipSuccess ||
+            n <= 0)
+            n = 2;
+        return n;
+    }();
+    const int resident = device_cu_count() * blocks_per_cu;
+    const dim3 grid(a.total_rows < resident ? a.total_rows : resident);
+    hipLaunchKernelGGL(update_rows_long_kernel<WITH_GS>, grid, dim3(kThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
+constexpr int kLongClass = 2000;
+
 template <int J, int W>
 hipError_t launch_split(hipStream_t stream, const BatchArgs& a) {
     return a.lr_scale != 0.0f ? launch_split_variant<J, W, true>(stream, a) : launch_split_variant<J, W, false>(stream, a);
@@ -518,8 +619,8 @@ hipError_t launch_iters(hipStream_t stream, const BatchArgs& a) {
 }
 
 // Row lengths (in units of 64 groups = 256 weights, rounded up) with a one-wave
-// register-resident variant: every length up to 4096 weights.  Longer rows, up to 22528
-// weights, are shared by four or eight waves; anything beyond takes the streamed row.
+// register-resident variant: every length up to 4096 weights.  Longer rows are read twice by
+// one wave, except 8192 < length <= 11264, which four waves share register-resident.
 #ifdef MCC_EXPERIMENT_FEW_VARIANTS
 #define MCC_RESIDENT_ITERS(X) X(3) X(8) X(16)
 #else
@@ -535,9 +636,6 @@ int iters_class(const UpdateTensor& t) {
     const int iters = ((t.in_features >> 2) + kWave - 1) / kWave;
     const bool aligned = (reinterpret_cast<uintptr_t>(t.grad_w) & 15u) == 0;
     if (!aligned) return 0;
-#ifdef MCC_EXPERIMENT_SPLIT16
-    if (iters > 8 && iters <= 16) return split_class(8, 2);
-#endif
     switch (iters) {
 #define MCC_CASE(N) case N:
         MCC_RESIDENT_ITERS(MCC_CASE)
@@ -545,10 +643,12 @@ int iters_class(const UpdateTensor& t) {
         return iters;
         default: break;
     }
-    if (iters > 16 && iters <= 24) return split_class(6, 4);
-    if (iters > 24 && iters <= 32) return split_class(8, 4);
+    // 11008-wide rows (the 7B FFN width) stay with four cooperating waves, which read the row
+    // once; every other long row takes the two-pass wave (measured at 4096 rows: 5120-wide 639
+    // against 425 Gweights/s for the cooperating waves, 8192-wide 664 against 604, 14336-wide 591
+    // against 300, 11008-wide 640 either way)
     if (iters > 32 && iters <= 44) return split_class(11, 4);
-    if (iters > 44 && iters <= 88) return split_class(11, 8);
+    if (iters > 16) return kLongClass;
     return 0;
 }
 
@@ -557,13 +657,9 @@ hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
 #define MCC_CASE(N) case N: return launch_iters<N>(stream, a);
         MCC_RESIDENT_ITERS(MCC_CASE)
 #undef MCC_CASE
-#ifdef MCC_EXPERIMENT_SPLIT16
-        case split_class(8, 2): return launch_split<8, 2>(stream, a);
-#endif
-        case split_class(6, 4): return launch_split<6, 4>(stream, a);
-        case split_class(8, 4): return launch_split<8, 4>(stream, a);
+        case kLongClass:
+            return a.lr_scale != 0.0f ? launch_long_variant<true>(stream, a) : launch_long_variant<false>(stream, a);
         case split_class(11, 4): return launch_split<11, 4>(stream, a);
-        case split_class(11, 8): return launch_split<11, 8>(stream, a);
         default: return launch_iters<0>(stream, a);
     }
 }
