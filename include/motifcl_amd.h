@@ -203,6 +203,12 @@ int mcc_compact_counter_decode_weight(
 /*
  * out[batch,out] = x[batch,in] . W(state)^T with the ternary weights decoded
  * from the packed state inside the contraction (no dense weight buffer).
+ * Runs on the bf16 matrix cores with every product exact: the ternary weight
+ * is exact in bf16 and each activation is split into three bf16 terms whose sum
+ * is the activation, so the result has fp32 accuracy (the terms of an fp32
+ * contraction, summed in another order).  Activations must be finite and
+ * below 3.38e38 in magnitude (the largest bf16); terms below 2^-110 lose
+ * their low bits.
  * Replaces run_vulkan_compact_counter_forward_u8
  * (include/motifcl/runtime/vulkan_backend.hpp:722-730,
  *  src/runtime/vulkan_backend.cpp:8662-8725).
@@ -216,7 +222,9 @@ int mcc_compact_counter_forward_u8(
     size_t batch, size_t in_features, size_t out_features, size_t C);
 
 /*
- * grad_x[batch,in] = grad_out[batch,out] . W(state), decoded in-kernel.
+ * grad_x[batch,in] = grad_out[batch,out] . W(state), decoded in-kernel; grad_out
+ * is multiplied by the row scale first, as the reference does, then split as in
+ * the forward product (same accuracy, same requirement of finite inputs).
  * Replaces run_vulkan_compact_counter_backward_input_u8
  * (include/motifcl/runtime/vulkan_backend.hpp:750-758,
  *  src/runtime/vulkan_backend.cpp:8727-8803; kernels/compact_counter.cl:248-269).
