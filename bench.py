@@ -133,7 +133,7 @@ def at_clock(roofline, mhz):
     return roofline
 
 
-def bench_fused(L, ops, name, steps, warmup, fused_path="workspace", graph=False):
+def bench_fused(L, ops, name, steps, warmup, fused_path="workspace", graph=False, batched=False):
     import torch
     desc, shapes, layers, tokens = WORKLOADS[name]
     gen = torch.Generator(device="cuda")
@@ -161,6 +161,18 @@ def bench_fused(L, ops, name, steps, warmup, fused_path="workspace", graph=False
         for k, ((state, scale, v), dy, x, n_out, n_in) in enumerate(tensors):
             ops.apply_update_fused(state, scale, v, dy, x, ws, C, LR, LR_SCALE, BETA, EPS,
                                    12345 + k + 1000 * i)
+
+    if batched:
+        # all tensors of the step in one call: grouped contraction, grouped slice sum, batched update
+        fb = ops.FusedBatch([(st[0], st[1], st[2], dy, x) for (st, dy, x, _, _) in tensors], LR,
+                            [12345 + k for k in range(len(tensors))])
+        ws_bytes = fb.workspace_nbytes()
+        del ws
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+
+        def step(i):  # noqa: F811
+            fb.set_seeds([12345 + k + 1000 * i for k in range(len(tensors))])
+            ops.apply_update_fused_batched(fb, ws, C, LR_SCALE, BETA, EPS)
 
     for i in range(warmup):
         step(i)
@@ -205,7 +217,8 @@ def bench_fused(L, ops, name, steps, warmup, fused_path="workspace", graph=False
                      "launches": gemm_n, "avg_launch_ms": gemm_ms / max(gemm_n, 1),
                      "algorithmic_flops_per_step": flops},
         "kernel_ms_per_step": {kernel: gemm_ms / steps, "counter_update": upd_ms / steps},
-        "fused_path": fused_path, "workspace_bytes": ws_bytes, "graph_replay_ms_per_step": graph_ms,
+        "fused_path": fused_path, "batched_call": batched, "workspace_bytes": ws_bytes,
+        "graph_replay_ms_per_step": graph_ms,
     }
     # the clock the dominant kernel runs at (the power limit holds it below the 2400 MHz of the
     # published peak): contraction alone on the two-kernel path, the whole step on the strip path
@@ -501,6 +514,8 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="also time the fused step captured into a HIP graph and replayed (reported beside "
                          "the eager figure, which stays the headline)")
+    ap.add_argument("--batched", action="store_true",
+                    help="fused leg through mcc_compact_counter_apply_update_fused_batched (one call per step)")
     ap.add_argument("--no-update-only", action="store_true", help="skip the cfg3 update-only leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-clock", action="store_true",
@@ -534,7 +549,8 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
-    fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup, args.fused_path, args.graph)
+    fused, fused_sample, tokens = bench_fused(L, ops, args.workload, args.steps, args.warmup, args.fused_path, args.graph,
+                                              args.batched)
     line = {
         "metric": "counter-synapse updates/s (Gparam/s)",
         "value": fused["value"], "unit": "Gparam/s", "n_gpus": 1, "steps": args.steps,

@@ -155,6 +155,39 @@ int mcc_compact_counter_apply_update_fused(
     float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
 
 /*
+ * The fused step for a list of tensors in a handful of launches: one grouped
+ * contraction per tile size, one launch that adds the token-chunk slices, and
+ * the batched update.  For models made of small layers (the 288- and 768-wide
+ * linears of the 15M-parameter model) the per-tensor entry point is bound by
+ * its three launches per tensor; this one costs about five launches for all of
+ * them.  It has no single counterpart in the reference: it stands for the
+ * per-layer calls of apply_update_backward (src/nn/compact_counter.cpp:158-231)
+ * of a caller that keeps every layer's grad_out and x alive until the end of
+ * its backward pass, which is equivalent because no layer's update reads
+ * another layer's state.  state, scale and v come out bit-identical to calling
+ * mcc_compact_counter_apply_update_fused per tensor with a full workspace.
+ * `workspace` (256-byte aligned) holds
+ * mcc_compact_counter_fused_batched_workspace_nbytes(tensors, n) bytes: the
+ * per-tensor workspaces, each rounded up to 256 bytes, one after the other.
+ * Under MCC_CONTRACTION_BF16X6 the tensors are processed one by one.
+ */
+typedef struct mcc_fused_tensor {
+    uint8_t* state;        size_t state_nbytes;
+    float* scale;          size_t scale_nbytes;
+    float* v;              size_t v_nbytes;
+    const float* grad_out; size_t grad_out_nbytes;  /* [batch, out_features] */
+    const float* x;        size_t x_nbytes;         /* [batch, in_features] */
+    size_t in_features, out_features, batch;
+    float lr;
+    uint32_t seed;
+} mcc_fused_tensor;
+size_t mcc_compact_counter_fused_batched_workspace_nbytes(const mcc_fused_tensor* tensors, size_t n_tensors);
+int mcc_compact_counter_apply_update_fused_batched(
+    void* stream, const mcc_fused_tensor* tensors, size_t n_tensors,
+    void* workspace, size_t workspace_nbytes,
+    size_t C, float lr_scale, float rms_beta, float rms_eps);
+
+/*
  * How the weight-gradient contraction (inside the two-kernel fused step and in
  * mcc_matmul_transpose_a_f32) multiplies.  Process-wide; no counterpart in the
  * reference.

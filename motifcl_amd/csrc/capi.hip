@@ -338,6 +338,109 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
     return MCC_OK;
 }
 
+// Where tensor i's slices start in a batched fused workspace: each tensor gets what
+// mcc_compact_counter_fused_workspace_nbytes asks for, rounded up to 256 bytes.
+static size_t fused_batched_region(const mcc_fused_tensor& t) {
+    const size_t full = mcc_compact_counter_fused_workspace_nbytes(t.in_features, t.out_features, t.batch);
+    return full == 0 ? 0 : (full + 255) / 256 * 256;
+}
+
+size_t mcc_compact_counter_fused_batched_workspace_nbytes(const mcc_fused_tensor* tensors, size_t n_tensors) {
+    if (!tensors) return 0;
+    size_t total = 0;
+    for (size_t i = 0; i < n_tensors; ++i) {
+        const size_t r = fused_batched_region(tensors[i]);
+        if (r == 0 || r > std::numeric_limits<size_t>::max() - total) return 0;
+        total += r;
+    }
+    return total;
+}
+
+int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused_tensor* tensors, size_t n_tensors,
+                                                   void* workspace, size_t workspace_nbytes, size_t C,
+                                                   float lr_scale, float rms_beta, float rms_eps) {
+    if (n_tensors == 0) return MCC_OK;
+    if (!tensors) return fail(MCC_E_INVALID, "compact-counter fused update received a null tensor list");
+    if (!workspace) return fail(MCC_E_INVALID, "compact-counter fused update received a null buffer");
+    if (reinterpret_cast<uintptr_t>(workspace) % 256)
+        return fail(MCC_E_INVALID, "compact-counter batched fused update workspace must be 256-byte aligned");
+    const size_t need = mcc_compact_counter_fused_batched_workspace_nbytes(tensors, n_tensors);
+    if (need == 0) return fail(MCC_E_INVALID, "compact-counter fused update requires non-zero dimensions");
+    if (workspace_nbytes < need) return fail(MCC_E_INVALID, "compact-counter fused update workspace is too small");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // another contraction mode than the fp32 instruction: tensor by tensor, each in its own region
+    if (g_contraction_mode.load() != MCC_CONTRACTION_FP32) {
+        uint8_t* ws = static_cast<uint8_t*>(workspace);
+        for (size_t i = 0; i < n_tensors; ++i) {
+            const mcc_fused_tensor& t = tensors[i];
+            const size_t region = fused_batched_region(t);
+            const int rc = mcc_compact_counter_apply_update_fused(
+                stream, t.state, t.state_nbytes, t.scale, t.scale_nbytes, t.v, t.v_nbytes, t.grad_out, t.grad_out_nbytes,
+                t.x, t.x_nbytes, ws, region, C, t.in_features, t.out_features, t.batch, t.lr, lr_scale, rms_beta,
+                rms_eps, t.seed);
+            if (rc != MCC_OK) {
+                g_error = "tensor " + std::to_string(i) + ": " + g_error;
+                return rc;
+            }
+            ws += region;
+        }
+        return MCC_OK;
+    }
+    std::vector<mcc::GemmTnJob> jobs(n_tensors);
+    std::vector<mcc::UpdateTensor> upd(n_tensors);
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    for (size_t i = 0; i < n_tensors; ++i) {
+        const mcc_fused_tensor& t = tensors[i];
+        const char* what = "compact-counter fused update";
+        int rc = MCC_OK;
+        if (t.batch == 0 || t.batch > kIntMax)
+            rc = fail(MCC_E_INVALID, "compact-counter fused update batch must be in [1, 2^31-1]");
+        else if (!check_codec(what, C, t.in_features, t.out_features))
+            rc = MCC_E_INVALID;
+        else if (!t.grad_out || !t.x)
+            rc = fail(MCC_E_INVALID, "compact-counter fused update received a null buffer");
+        else if (t.batch > std::numeric_limits<size_t>::max() / sizeof(float) / t.in_features ||
+                 t.batch > std::numeric_limits<size_t>::max() / sizeof(float) / t.out_features)
+            rc = fail(MCC_E_INVALID, "compact-counter fused update activation size overflows size_t");
+        else if (t.grad_out_nbytes < t.batch * t.out_features * sizeof(float) ||
+                 t.x_nbytes < t.batch * t.in_features * sizeof(float))
+            rc = fail(MCC_E_INVALID, "compact-counter fused update activation buffer is too small");
+        else if (reinterpret_cast<uintptr_t>(t.grad_out) % alignof(float) || reinterpret_cast<uintptr_t>(t.x) % alignof(float))
+            rc = fail(MCC_E_INVALID, "compact-counter fused update float buffers must be 4-byte aligned");
+        if (rc == MCC_OK) {
+            // the state side is checked as for the update-only step, with the tensor's region as gradient
+            const mcc_counter_tensor c = {t.state, t.state_nbytes, t.scale, t.scale_nbytes, t.v, t.v_nbytes,
+                                          reinterpret_cast<const float*>(ws),
+                                          t.out_features * t.in_features * sizeof(float), t.in_features,
+                                          t.out_features, t.lr, t.seed};
+            rc = check_update_tensor(c, C, lr_scale, rms_beta, rms_eps, &upd[i]);
+        }
+        if (rc != MCC_OK) {
+            g_error = "tensor " + std::to_string(i) + ": " + g_error;
+            return rc;
+        }
+        jobs[i].a = t.grad_out;
+        jobs[i].b = t.x;
+        jobs[i].out = reinterpret_cast<float*>(ws);
+        jobs[i].k = (int)t.batch;
+        jobs[i].m = (int)t.out_features;
+        jobs[i].n = (int)t.in_features;
+        ws += fused_batched_region(t);
+    }
+    hipError_t e;
+    {
+        ScopedKernelTimer timer("gemm_tn_f32", s);
+        e = mcc::launch_gemm_tn_group(s, jobs.data(), n_tensors);
+    }
+    if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
+    {
+        ScopedKernelTimer timer("counter_update", s);
+        e = mcc::launch_update_batch(s, upd.data(), n_tensors, (int)C, lr_scale, rms_beta, rms_eps);
+    }
+    if (e != hipSuccess) return hip_fail(e, "compact-counter fused update launch failed");
+    return MCC_OK;
+}
+
 int mcc_set_contraction_mode(int mode) {
     if (mode != MCC_CONTRACTION_FP32 && mode != MCC_CONTRACTION_BF16X6)
         return fail(MCC_E_INVALID, "unknown contraction mode");

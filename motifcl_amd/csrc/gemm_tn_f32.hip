@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <vector>
 
 #include "gemm_tile.hpp"
 #include "launch.hpp"
@@ -55,6 +56,85 @@ __global__ __launch_bounds__(256) void reduce_slices_kernel(const float* __restr
         float acc = slices[e];
         for (int s = 1; s < n_slices; ++s) acc = acc + slices[(size_t)s * mn + e];
         c[e] = acc;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Grouped form: the contractions of several tensors in one launch (and one launch that adds
+// their chunk slices).  A small layer is tens of microseconds of work, so a model made of such
+// layers is bound by launches when every tensor goes out on its own; here the descriptors
+// travel as kernel arguments and a workgroup finds its tensor by scanning their first-workgroup
+// indices.  Each tensor keeps the plan (tile size, chunks) it has on its own, and the register-
+// staged main loop sums in the same order as the direct-to-LDS one, so the gradients are the
+// same bits as from launch_gemm_tn_f32.
+// ---------------------------------------------------------------------------
+struct GemmGroupItem {
+    const float* a;
+    const float* b;
+    float* out;  // slice 0 (the chunk slices are M*N floats apart)
+    int K, M, N, chunk, tiles_x, tiles, wg_start, pad;
+};
+constexpr int kMaxGemmGroup = 56;  // 56 descriptors of 56 bytes: the kernel arguments stay below 4 KiB
+struct GemmGroupArgs {
+    GemmGroupItem it[kMaxGemmGroup];
+    int n;
+};
+
+template <int BM, int BN>
+__global__ __launch_bounds__(kGemmThreads) void gemm_tn_group_kernel(GemmGroupArgs g) {
+    using Cfg = TileCfg<BM, BN>;
+    __shared__ float lds[Cfg::kLdsFloats];
+    const int wg = blockIdx.x;
+    int i = 0;
+    while (i + 1 < g.n && wg >= g.it[i + 1].wg_start) ++i;  // uniform: scalar loads of the arguments
+    const GemmGroupItem it = g.it[i];
+    const int local = wg - it.wg_start;
+    const int z = local / it.tiles, t = local - z * it.tiles;
+    const int ty = t / it.tiles_x, tx = t - ty * it.tiles_x;
+    const TilePos tp = tile_pos<BM, BN>();
+    const int m0 = ty * BM, n0 = tx * BN;
+    const int k_begin = z * it.chunk;
+    const int k_len = it.K - k_begin < it.chunk ? it.K - k_begin : it.chunk;
+    const float* a = it.a + (size_t)k_begin * it.M;
+    const float* b = it.b + (size_t)k_begin * it.N;
+    float* c = it.out + (size_t)z * it.M * it.N;
+    floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
+    gemm_tile_mainloop<BM, BN, true, true>(a, b, k_len, it.M, it.N, m0, n0, tp, lds, acc);
+#pragma unroll
+    for (int ii = 0; ii < Cfg::kTilesM; ++ii)
+#pragma unroll
+        for (int j = 0; j < Cfg::kTilesN; ++j) {
+            const int col = n0 + tp.wn0 + 32 * j + tp.l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + tp.wm0 + 32 * ii + 8 * (r / 4) + 4 * tp.half + (r % 4);
+                if (row < it.M && col < it.N) c[(size_t)row * it.N + col] = acc[ii][j][r];
+            }
+        }
+}
+
+struct ReduceGroupItem {
+    float* slices;  // summed in place into slice 0
+    unsigned mn;
+    int n_slices, block_start, pad;
+};
+constexpr int kMaxReduceGroup = 128;
+struct ReduceGroupArgs {
+    ReduceGroupItem it[kMaxReduceGroup];
+    int n;
+};
+constexpr int kReduceBlockElems = 256;  // one element per thread: a thread's chunk loads are all in flight at once
+
+__global__ __launch_bounds__(256) void reduce_slices_group_kernel(ReduceGroupArgs g) {
+    const int wg = blockIdx.x;
+    int i = 0;
+    while (i + 1 < g.n && wg >= g.it[i + 1].block_start) ++i;
+    const ReduceGroupItem it = g.it[i];
+    const unsigned e = (unsigned)(wg - it.block_start) * kReduceBlockElems + threadIdx.x;
+    if (e < it.mn) {
+        float acc = it.slices[e];
+        for (int s = 1; s < it.n_slices; ++s) acc = acc + it.slices[(size_t)s * it.mn + e];
+        it.slices[e] = acc;
     }
 }
 
@@ -128,6 +208,88 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
     hipLaunchKernelGGL(reduce_slices_kernel, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, stream, slices,
                        c, mn, plan.splits);
     return hipGetLastError();
+}
+
+// The contractions of `n` tensors (c = slice 0 of `out`, which holds gemm_tn_slices floats-matrices).
+// Tensors whose operands are 16-byte aligned with m, n multiples of 4 are grouped by tile size;
+// the others, and very large ones (which fill the device alone), go out one by one.
+hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_t n) {
+    std::vector<char> grouped(n, 0);
+    for (int tile : {64, 128}) {
+        GemmGroupArgs g;
+        g.n = 0;
+        int wgs = 0;
+        auto flush = [&]() -> hipError_t {
+            if (g.n == 0) return hipSuccess;
+            if (tile == 64)
+                hipLaunchKernelGGL((gemm_tn_group_kernel<64, 64>), dim3(wgs), dim3(kGemmThreads), 0, stream, g);
+            else
+                hipLaunchKernelGGL((gemm_tn_group_kernel<128, 128>), dim3(wgs), dim3(kGemmThreads), 0, stream, g);
+            g.n = 0;
+            wgs = 0;
+            return hipGetLastError();
+        };
+        for (size_t i = 0; i < n; ++i) {
+            const GemmTnJob& j = jobs[i];
+            const GemmTnPlan plan = plan_gemm_tn(j.k, j.m, j.n);
+            const bool vec = j.m % 4 == 0 && j.n % 4 == 0 && (reinterpret_cast<uintptr_t>(j.a) & 15u) == 0 &&
+                             (reinterpret_cast<uintptr_t>(j.b) & 15u) == 0;
+            const long tiles = (long)((j.m + plan.tile - 1) / plan.tile) * ((j.n + plan.tile - 1) / plan.tile);
+            // a tensor of 1024 workgroups or more gains nothing from sharing a launch
+            if (plan.tile != tile || !vec || tiles * plan.splits >= 1024) continue;
+            if (g.n == kMaxGemmGroup || wgs > (1 << 30)) {
+                const hipError_t e = flush();
+                if (e != hipSuccess) return e;
+            }
+            GemmGroupItem& it = g.it[g.n++];
+            it.a = j.a; it.b = j.b; it.out = j.out;
+            it.K = j.k; it.M = j.m; it.N = j.n;
+            it.chunk = plan.chunk;
+            it.tiles_x = (j.n + tile - 1) / tile;
+            it.tiles = (int)tiles;
+            it.wg_start = wgs;
+            it.pad = 0;
+            wgs += (int)tiles * plan.splits;
+            grouped[i] = 1;
+        }
+        const hipError_t e = flush();
+        if (e != hipSuccess) return e;
+    }
+    // the rest one by one (this also adds their slices)
+    for (size_t i = 0; i < n; ++i) {
+        if (grouped[i]) continue;
+        const hipError_t e = launch_gemm_tn_f32(stream, jobs[i].a, jobs[i].b, jobs[i].out, jobs[i].k, jobs[i].m,
+                                                jobs[i].n, jobs[i].out, 0);
+        if (e != hipSuccess) return e;
+    }
+    // slices of the grouped tensors, in chunk order
+    ReduceGroupArgs r;
+    r.n = 0;
+    int blocks = 0;
+    auto flush_reduce = [&]() -> hipError_t {
+        if (r.n == 0) return hipSuccess;
+        hipLaunchKernelGGL(reduce_slices_group_kernel, dim3(blocks), dim3(256), 0, stream, r);
+        r.n = 0;
+        blocks = 0;
+        return hipGetLastError();
+    };
+    for (size_t i = 0; i < n; ++i) {
+        if (!grouped[i]) continue;
+        const GemmTnPlan plan = plan_gemm_tn(jobs[i].k, jobs[i].m, jobs[i].n);
+        if (plan.splits == 1) continue;
+        if (r.n == kMaxReduceGroup) {
+            const hipError_t e = flush_reduce();
+            if (e != hipSuccess) return e;
+        }
+        ReduceGroupItem& it = r.it[r.n++];
+        it.slices = jobs[i].out;
+        it.mn = (unsigned)((size_t)jobs[i].m * jobs[i].n);  // below 2^32: the tensor has fewer than 1024 tiles
+        it.n_slices = plan.splits;
+        it.block_start = blocks;
+        it.pad = 0;
+        blocks += (int)((it.mn + kReduceBlockElems - 1) / kReduceBlockElems);
+    }
+    return flush_reduce();
 }
 
 }  // namespace mcc

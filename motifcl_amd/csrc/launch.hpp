@@ -44,6 +44,16 @@ size_t gemm_tn_slices(int k, int m, int n);
 // passes (gemm_tn_bf16x6.hip), where the shape allows it
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c,
                               int k, int m, int n, float* slices, int mode = 0);
+// One contraction of a grouped launch: out holds gemm_tn_slices(k, m, n) matrices of m*n floats,
+// the result ends up in the first.
+struct GemmTnJob {
+    const float* a;  // [k, m]
+    const float* b;  // [k, n]
+    float* out;
+    int k, m, n;
+};
+hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_t n);
+
 bool gemm_tn_bf16x6_supports(const float* a, const float* b, int k, int m, int n, const GemmTnPlan& plan);
 hipError_t launch_gemm_tn_bf16x6(hipStream_t stream, const float* a, const float* b, float* out,
                                  int k, int m, int n, const GemmTnPlan& plan);

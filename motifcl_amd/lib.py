@@ -22,6 +22,9 @@ SIGNATURES = {
     "mcc_compact_counter_apply_update_fused": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
                        _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
+    "mcc_compact_counter_fused_batched_workspace_nbytes": (_sz, [_vp, _sz]),
+    "mcc_compact_counter_apply_update_fused_batched": (
+        ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _f, _f, _f]),
     "mcc_set_contraction_mode": (ctypes.c_int, [ctypes.c_int]),
     "mcc_get_contraction_mode": (ctypes.c_int, []),
     "mcc_matmul_transpose_a_f32": (ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _sz, _sz, _sz]),
@@ -58,6 +61,14 @@ class CounterTensor(ctypes.Structure):
     _fields_ = [("state", _vp), ("state_nbytes", _sz), ("scale", _vp), ("scale_nbytes", _sz),
                 ("v", _vp), ("v_nbytes", _sz), ("grad_w", _vp), ("grad_w_nbytes", _sz),
                 ("in_features", _sz), ("out_features", _sz), ("lr", _f), ("seed", _u32)]
+
+
+class FusedTensor(ctypes.Structure):
+    """struct mcc_fused_tensor of include/motifcl_amd.h."""
+    _fields_ = [("state", _vp), ("state_nbytes", _sz), ("scale", _vp), ("scale_nbytes", _sz),
+                ("v", _vp), ("v_nbytes", _sz), ("grad_out", _vp), ("grad_out_nbytes", _sz),
+                ("x", _vp), ("x_nbytes", _sz), ("in_features", _sz), ("out_features", _sz),
+                ("batch", _sz), ("lr", _f), ("seed", _u32)]
 
 
 _lib = None

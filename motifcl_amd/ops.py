@@ -66,6 +66,42 @@ def apply_update_dense_batched(batch, C, lr_scale, rms_beta, rms_eps):
         _stream(), batch.array, batch.n, C, lr_scale, rms_beta, rms_eps))
 
 
+class FusedBatch:
+    """A reusable descriptor list for apply_update_fused_batched: tensors are
+    (state, scale, v, grad_out [batch, out], x [batch, in]) device tensors."""
+
+    def __init__(self, tensors, lr, seeds):
+        self._keep = list(tensors)
+        n = len(self._keep)
+        self.array = (_lib.FusedTensor * n)()
+        for i, (state, scale, v, grad_out, x) in enumerate(self._keep):
+            batch, out_features = grad_out.shape
+            d = self.array[i]
+            d.state, d.state_nbytes = _buf(state, torch.uint8)
+            d.scale, d.scale_nbytes = _buf(scale, torch.float32)
+            d.v, d.v_nbytes = _buf(v, torch.float32)
+            d.grad_out, d.grad_out_nbytes = _buf(grad_out, torch.float32)
+            d.x, d.x_nbytes = _buf(x, torch.float32)
+            d.in_features, d.out_features, d.batch = x.shape[1], out_features, batch
+            d.lr = lr[i] if isinstance(lr, (list, tuple)) else lr
+            d.seed = seeds[i] & 0xFFFFFFFF
+        self.n = n
+
+    def set_seeds(self, seeds):
+        for i in range(self.n):
+            self.array[i].seed = seeds[i] & 0xFFFFFFFF
+
+    def workspace_nbytes(self):
+        return int(_lib.load().mcc_compact_counter_fused_batched_workspace_nbytes(self.array, self.n))
+
+
+def apply_update_fused_batched(batch, workspace, C, lr_scale, rms_beta, rms_eps):
+    """In-place fused step of every tensor of a FusedBatch in a handful of launches."""
+    L = _lib.load()
+    _lib.check(L.mcc_compact_counter_apply_update_fused_batched(
+        _stream(), batch.array, batch.n, *_buf(workspace, torch.uint8), C, lr_scale, rms_beta, rms_eps))
+
+
 def fused_workspace_nbytes(in_features, out_features, batch):
     return int(_lib.load().mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch))
 
