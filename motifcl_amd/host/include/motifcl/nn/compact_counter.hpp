@@ -4,6 +4,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <vector>
 
 #include <motifcl/nn/module.hpp>
 #include <motifcl/runtime/backend.hpp>
@@ -21,6 +22,34 @@ namespace motifcl::nn {
 //   Auto   Strip for layers of at least 128 tiles of 128 x 128 (2M weights), Full below
 // All give identical bytes.
 enum class FusedWorkspace { Auto, Strip, Full };
+
+class CounterStateLinear;
+
+// Collects the fused updates of a backward pass and applies them in one batched call
+// (mcc_compact_counter_apply_update_fused_batched): models made of small layers are bound by the
+// three launches per layer of the immediate update.  Not in the reference, whose
+// CounterBackwardNode updates at once (src/nn/compact_counter.cpp:30-51); the results are the
+// same bytes, because no layer's update reads another layer's state and grad_x is taken from the
+// pre-update state either way.  The recorded grad_out and x stay alive until flush().
+//
+//     DeferredCounterUpdates pending;
+//     for (auto* l : layers) l->set_deferred(&pending);
+//     loss.backward();          // records (layer, grad_out, x, seed) per layer
+//     pending.flush();          // one call for all of them
+class DeferredCounterUpdates {
+public:
+    void add(CounterStateLinear& layer, const Tensor& grad_out, const Tensor& x, std::uint32_t seed);
+    void flush();
+    std::size_t size() const { return items_.size(); }
+
+private:
+    struct Item {
+        CounterStateLinear* layer;
+        Tensor grad_out, x;
+        std::uint32_t seed;
+    };
+    std::vector<Item> items_;
+};
 
 // Ternary finite-state "counter" linear layer trained as a per-synapse automaton: the whole
 // trainable state is a packed 6-bit code per weight plus a per-row scale and a per-row RMS
@@ -46,6 +75,9 @@ public:
     void set_training(bool t) { training_ = t; }
     bool training() const { return training_; }
     void set_fused_workspace(FusedWorkspace w) { fused_workspace_ = w; }
+    // With a collector set, backward records the update instead of applying it (see above).
+    void set_deferred(DeferredCounterUpdates* d) { deferred_ = d; }
+    DeferredCounterUpdates* deferred() const { return deferred_; }
     FusedWorkspace fused_workspace() const { return fused_workspace_; }
     // Waits for the backend and throws if the last Strip update gave up an inter-tile wait.
     void check_fused_update() const;
@@ -72,6 +104,8 @@ private:
     std::uint32_t seed_ = 12345u;
     bool training_ = true;
     FusedWorkspace fused_workspace_ = FusedWorkspace::Auto;
+    DeferredCounterUpdates* deferred_ = nullptr;
+    friend class DeferredCounterUpdates;
     std::size_t last_fused_ws_ = 0, last_fused_batch_ = 0;
 };
 

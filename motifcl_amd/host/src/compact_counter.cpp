@@ -39,7 +39,10 @@ struct CounterBackwardNode : autograd::Node {
         if (need_gx) grad_x = layer->backward_input_from_state(grad_out);  // PRE-update state
         {
             autograd::NoGradGuard guard;
-            layer->apply_update_backward(grad_out, x, seed);
+            if (layer->deferred())
+                layer->deferred()->add(*layer, grad_out, x, seed);
+            else
+                layer->apply_update_backward(grad_out, x, seed);
         }
         if (need_gx) x.backward(grad_x);
     }
@@ -120,6 +123,53 @@ void CounterStateLinear::apply_update_backward(const Tensor& grad_out, const Ten
     MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter fused update failed: ") + mcc_last_error());
     last_fused_ws_ = ws;
     last_fused_batch_ = N;
+}
+
+void DeferredCounterUpdates::add(CounterStateLinear& layer, const Tensor& grad_out, const Tensor& x,
+                                 std::uint32_t seed) {
+    MCL_CHECK(x.ndim() == 2 && grad_out.ndim() == 2, "apply_update_backward expects rank-2 tensors");
+    MCL_CHECK(items_.empty() || items_.front().layer->backend_ == layer.backend_,
+              "DeferredCounterUpdates collects layers of one backend");
+    MCL_CHECK(items_.empty() || (items_.front().layer->C_ == layer.C_ && items_.front().layer->lr_scale_ == layer.lr_scale_ &&
+                                 items_.front().layer->rms_beta_ == layer.rms_beta_ &&
+                                 items_.front().layer->rms_eps_ == layer.rms_eps_),
+              "DeferredCounterUpdates collects layers with the same C, lr_scale, rms_beta and rms_eps");
+    items_.push_back(Item{&layer, grad_out, x, seed});
+}
+
+void DeferredCounterUpdates::flush() {
+    if (items_.empty()) return;
+    std::vector<mcc_fused_tensor> list(items_.size());
+    for (std::size_t i = 0; i < items_.size(); ++i) {
+        Item& it = items_[i];
+        CounterStateLinear& l = *it.layer;
+        mcc_fused_tensor& t = list[i];
+        t.state = static_cast<std::uint8_t*>(l.state.data());
+        t.state_nbytes = l.state.nbytes();
+        t.scale = f32(l.scale);
+        t.scale_nbytes = l.scale.nbytes();
+        t.v = f32(l.v);
+        t.v_nbytes = l.v.nbytes();
+        t.grad_out = f32(it.grad_out);
+        t.grad_out_nbytes = it.grad_out.nbytes();
+        t.x = f32(it.x);
+        t.x_nbytes = it.x.nbytes();
+        t.in_features = static_cast<std::size_t>(l.in_);
+        t.out_features = static_cast<std::size_t>(l.out_);
+        t.batch = static_cast<std::size_t>(it.x.shape()[0]);
+        t.lr = l.lr_;
+        t.seed = it.seed;
+    }
+    CounterStateLinear& first = *items_.front().layer;
+    const std::size_t ws = mcc_compact_counter_fused_batched_workspace_nbytes(list.data(), list.size());
+    MCL_CHECK(ws != 0, "hip compact-counter fused update failed: batched workspace size is zero");
+    void* scratch = first.backend_->workspace(ws);
+    const int rc = mcc_compact_counter_apply_update_fused_batched(
+        first.backend_->hip_stream(), list.data(), list.size(), scratch, ws, static_cast<std::size_t>(first.C_),
+        first.lr_scale_, first.rms_beta_, first.rms_eps_);
+    MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter fused update failed: ") + mcc_last_error());
+    for (Item& it : items_) it.layer->last_fused_ws_ = 0;  // nothing to check across workgroups on this path
+    items_.clear();  // releases grad_out and x (the stream keeps them until the kernels have run)
 }
 
 void CounterStateLinear::check_fused_update() const {

@@ -10,7 +10,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BUILD = os.path.join(ROOT, "motifcl_amd", "host", "build")
 TESTS = ["test_counter_fused", "test_counter_state", "test_memory_gate", "test_layer_errors",
-         "test_checkpoint", "test_adam"]
+         "test_checkpoint", "test_adam", "test_deferred_updates"]
 
 
 def _built():
