@@ -164,6 +164,17 @@ hipError_t launch_tile(hipStream_t stream, const float* a, const float* b, float
 
 }  // namespace
 
+// One 256 x 256 tile occupies a CU (8 waves, 64 KiB of LDS, 128 accumulator registers), so the
+// wide kernel only pays when the tiles come in whole rounds of the 256 CUs: 4096 x 4096 is
+// exactly one round (+4 % over 128 x 128 tiles), 11008 x 4096 is 2.69 rounds and loses 10 % to
+// the last one, where the small tiles lose 2 %.
+static bool wide_tiles_fill_the_device(int m, int n) {
+    if (m % 256 || n % 256) return false;
+    const long tiles = (long)(m / 256) * (n / 256);
+    const long rounds = (tiles + 255) / 256;
+    return tiles >= 256 && tiles * 100 >= rounds * 256 * 97;
+}
+
 // How a contraction is cut up is a function of its shape alone, so that every entry point that
 // contracts the same operands produces the same bits.  Output tiles are 128 x 128 when that
 // gives at least 64 tiles (measured: 2048 x 768 at 16384 tokens runs 15 % faster as 96 large tiles
@@ -199,6 +210,8 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
     hipError_t e;
     if (mode == 1 && gemm_tn_bf16x6_supports(a, b, k, m, n, plan))
         e = launch_gemm_tn_bf16x6(stream, a, b, out, k, m, n, plan);
+    else if (plan.tile == 128 && wide_tiles_fill_the_device(m, n) && gemm_tn_wide_supports(a, b, k, m, n, plan.chunk))
+        e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, plan.chunk, plan.splits);
     else
         e = plan.tile == 128 ? launch_tile<128, 128>(stream, a, b, out, k, m, n, plan)
                                     : launch_tile<64, 64>(stream, a, b, out, k, m, n, plan);

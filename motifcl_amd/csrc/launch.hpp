@@ -44,6 +44,11 @@ size_t gemm_tn_slices(int k, int m, int n);
 // passes (gemm_tn_bf16x6.hip), where the shape allows it
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c,
                               int k, int m, int n, float* slices, int mode = 0);
+// 256 x 256-tile form of the contraction for whole tiles (gemm_tn_f32_wide.hip)
+bool gemm_tn_wide_supports(const float* a, const float* b, int k, int m, int n, int chunk);
+hipError_t launch_gemm_tn_wide(hipStream_t stream, const float* a, const float* b, float* out, int k, int m, int n,
+                               int chunk, int splits);
+
 // One contraction of a grouped launch: out holds gemm_tn_slices(k, m, n) matrices of m*n floats,
 // the result ends up in the first.
 struct GemmTnJob {
