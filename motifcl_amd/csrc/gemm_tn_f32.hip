@@ -138,10 +138,12 @@ __global__ __launch_bounds__(256) void reduce_slices_group_kernel(ReduceGroupArg
     }
 }
 
+// tiles_x, tiles_y > 0 restrict the launch to that many tiles from a, b, c on (a corner block of
+// the matrix: m and n stay the row lengths)
 template <int BM, int BN>
 hipError_t launch_tile(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n,
-                       const GemmTnPlan& plan) {
-    const dim3 grid((n + BN - 1) / BN, (m + BM - 1) / BM, plan.splits);
+                       const GemmTnPlan& plan, int tiles_x = 0, int tiles_y = 0) {
+    const dim3 grid(tiles_x > 0 ? tiles_x : (n + BN - 1) / BN, tiles_y > 0 ? tiles_y : (m + BM - 1) / BM, plan.splits);
     // every chunk starts at a multiple of 16 tokens, so it is as aligned as the matrix itself
     const bool vec_a = (m % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15u) == 0);
     const bool vec_b = (n % 4 == 0) && ((reinterpret_cast<uintptr_t>(b) & 15u) == 0);
@@ -173,6 +175,18 @@ static bool wide_tiles_fill_the_device(int m, int n) {
     const long tiles = (long)(m / 256) * (n / 256);
     const long rounds = (tiles + 255) / 256;
     return tiles >= 256 && tiles * 100 >= rounds * 256 * 97;
+}
+
+// For a matrix of `lines` x `across` wide tiles that is more than one round but not whole rounds:
+// how many lines make whole rounds of 256 tiles (0: none do).  11008 x 4096 is 43 x 16 tiles:
+// 32 lines are two rounds, the other 11 lines go to the small tiles.
+static int wide_block(int lines, int across) {
+    const long tiles = (long)lines * across;
+    if (tiles <= 256 || across <= 0) return 0;
+    const long full = tiles / 256 * 256;
+    if (full % across) return 0;
+    const long block = full / across;
+    return block < lines ? (int)block : 0;
 }
 
 // How a contraction is cut up is a function of its shape alone, so that every entry point that
@@ -208,11 +222,26 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
     float* out = plan.splits > 1 ? slices : c;
     if (plan.splits > 1 && !slices) return hipErrorInvalidValue;
     hipError_t e;
+    int wide_rows = 0, wide_cols = 0;
     if (mode == 1 && gemm_tn_bf16x6_supports(a, b, k, m, n, plan))
         e = launch_gemm_tn_bf16x6(stream, a, b, out, k, m, n, plan);
     else if (plan.tile == 128 && wide_tiles_fill_the_device(m, n) && gemm_tn_wide_supports(a, b, k, m, n, plan.chunk))
-        e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, plan.chunk, plan.splits);
-    else
+        e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, n / 256, m / 256, plan.chunk, plan.splits);
+    else if (plan.tile == 128 && plan.splits == 1 && gemm_tn_wide_supports(a, b, k, m, n, plan.chunk) &&
+             (wide_rows = wide_block(m / 256, n / 256)) + (wide_cols = wide_block(n / 256, m / 256)) > 0) {
+        // whole rounds of wide tiles on a block of rows (or columns), small tiles on the rest
+        if (wide_rows > 0) {
+            const int r = 256 * wide_rows;
+            e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, n / 256, wide_rows, plan.chunk, 1);
+            if (e == hipSuccess)
+                e = launch_tile<128, 128>(stream, a + r, b, out + (size_t)r * n, k, m, n, plan, n / 128, (m - r) / 128);
+        } else {
+            const int cw = 256 * wide_cols;
+            e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, wide_cols, m / 256, plan.chunk, 1);
+            if (e == hipSuccess)
+                e = launch_tile<128, 128>(stream, a, b + cw, out + cw, k, m, n, plan, (n - cw) / 128, m / 128);
+        }
+    } else
         e = plan.tile == 128 ? launch_tile<128, 128>(stream, a, b, out, k, m, n, plan)
                                     : launch_tile<64, 64>(stream, a, b, out, k, m, n, plan);
     if (e != hipSuccess || plan.splits == 1) return e;

@@ -107,9 +107,10 @@ bool gemm_tn_wide_supports(const float* a, const float* b, int k, int m, int n, 
            (reinterpret_cast<uintptr_t>(a) & 15u) == 0 && (reinterpret_cast<uintptr_t>(b) & 15u) == 0;
 }
 
+// tiles_x x tiles_y tiles starting at a, b, out; m and n are the row lengths of a / b and out
 hipError_t launch_gemm_tn_wide(hipStream_t stream, const float* a, const float* b, float* out, int k, int m, int n,
-                               int chunk, int splits) {
-    const dim3 grid(n / kWide, m / kWide, splits);
+                               int tiles_x, int tiles_y, int chunk, int splits) {
+    const dim3 grid(tiles_x, tiles_y, splits);
     hipLaunchKernelGGL(gemm_tn_wide_kernel, grid, dim3(kWideThreads), 0, stream, a, b, out, k, m, n, chunk);
     return hipGetLastError();
 }

@@ -47,7 +47,7 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
 // 256 x 256-tile form of the contraction for whole tiles (gemm_tn_f32_wide.hip)
 bool gemm_tn_wide_supports(const float* a, const float* b, int k, int m, int n, int chunk);
 hipError_t launch_gemm_tn_wide(hipStream_t stream, const float* a, const float* b, float* out, int k, int m, int n,
-                               int chunk, int splits);
+                               int tiles_x, int tiles_y, int chunk, int splits);
 
 // One contraction of a grouped launch: out holds gemm_tn_slices(k, m, n) matrices of m*n floats,
 // the result ends up in the first.
