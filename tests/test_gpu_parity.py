@@ -184,7 +184,10 @@ def test_integer_ticks_closed_form_on_gpu(ops, oracle):
 
 
 GEMM_SHAPES = [(37, 35, 68), (2, 2, 8), (33, 7, 5), (4096, 288, 288), (1000, 768, 288),
-               (512, 288, 768), (640, 300, 1028), (256, 1024, 2048)]
+               (512, 288, 768), (640, 300, 1028), (256, 1024, 2048),
+               # 256 x 256 tiles: one whole round; two rounds of wide tiles + small tiles for the other
+               # rows, and the same split by columns; 3.5 rounds
+               (48, 4096, 4096), (32, 11008, 4096), (32, 4096, 11008), (16, 14336, 4096)]
 
 
 @pytest.mark.parametrize("kmn", GEMM_SHAPES, ids=lambda s: "k%d_m%d_n%d" % s)
