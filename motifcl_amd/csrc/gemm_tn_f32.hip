@@ -222,28 +222,29 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
     float* out = plan.splits > 1 ? slices : c;
     if (plan.splits > 1 && !slices) return hipErrorInvalidValue;
     hipError_t e;
-    int wide_rows = 0, wide_cols = 0;
-    if (mode == 1 && gemm_tn_bf16x6_supports(a, b, k, m, n, plan))
+    const bool wide_ok = plan.tile == 128 && gemm_tn_wide_supports(a, b, k, m, n, plan.chunk);
+    // rows or columns of wide tiles that make whole rounds, when the whole matrix does not
+    const int wide_rows = wide_ok && plan.splits == 1 ? wide_block(m / 256, n / 256) : 0;
+    const int wide_cols = wide_ok && plan.splits == 1 && wide_rows == 0 ? wide_block(n / 256, m / 256) : 0;
+    if (mode == 1 && gemm_tn_bf16x6_supports(a, b, k, m, n, plan)) {
         e = launch_gemm_tn_bf16x6(stream, a, b, out, k, m, n, plan);
-    else if (plan.tile == 128 && wide_tiles_fill_the_device(m, n) && gemm_tn_wide_supports(a, b, k, m, n, plan.chunk))
+    } else if (wide_ok && wide_tiles_fill_the_device(m, n)) {
         e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, n / 256, m / 256, plan.chunk, plan.splits);
-    else if (plan.tile == 128 && plan.splits == 1 && gemm_tn_wide_supports(a, b, k, m, n, plan.chunk) &&
-             (wide_rows = wide_block(m / 256, n / 256)) + (wide_cols = wide_block(n / 256, m / 256)) > 0) {
-        // whole rounds of wide tiles on a block of rows (or columns), small tiles on the rest
-        if (wide_rows > 0) {
-            const int r = 256 * wide_rows;
-            e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, n / 256, wide_rows, plan.chunk, 1);
-            if (e == hipSuccess)
-                e = launch_tile<128, 128>(stream, a + r, b, out + (size_t)r * n, k, m, n, plan, n / 128, (m - r) / 128);
-        } else {
-            const int cw = 256 * wide_cols;
-            e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, wide_cols, m / 256, plan.chunk, 1);
-            if (e == hipSuccess)
-                e = launch_tile<128, 128>(stream, a, b + cw, out + cw, k, m, n, plan, (n - cw) / 128, m / 128);
-        }
-    } else
+    } else if (wide_rows > 0) {
+        // wide tiles on the first rows, small tiles on the rest
+        const int r = 256 * wide_rows;
+        e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, n / 256, wide_rows, plan.chunk, 1);
+        if (e == hipSuccess)
+            e = launch_tile<128, 128>(stream, a + r, b, out + (size_t)r * n, k, m, n, plan, n / 128, (m - r) / 128);
+    } else if (wide_cols > 0) {
+        const int cw = 256 * wide_cols;
+        e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, wide_cols, m / 256, plan.chunk, 1);
+        if (e == hipSuccess)
+            e = launch_tile<128, 128>(stream, a, b + cw, out + cw, k, m, n, plan, (n - cw) / 128, m / 128);
+    } else {
         e = plan.tile == 128 ? launch_tile<128, 128>(stream, a, b, out, k, m, n, plan)
-                                    : launch_tile<64, 64>(stream, a, b, out, k, m, n, plan);
+                             : launch_tile<64, 64>(stream, a, b, out, k, m, n, plan);
+    }
     if (e != hipSuccess || plan.splits == 1) return e;
     const size_t mn = (size_t)m * n;
     const size_t want = (mn + 255) / 256;
