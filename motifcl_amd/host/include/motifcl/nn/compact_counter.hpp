@@ -16,7 +16,7 @@ namespace motifcl::nn {
 //          exchange 32 KiB of partial row sums (no weight-sized buffer, as in the reference,
 //          tests/test_memory_truth_gate.cpp:109-113); needs lr_scale == 0 and in/out multiples
 //          of 128, other layers silently use Full
-//   Full   contraction into f32[out,in] workspace slices, then the update kernel (a few percent
+//   Full   contraction into f32[out,in] workspace slices, then the update kernel (about 10 percent
 //          faster on large layers; the only way to keep the GPU busy on small ones, whose token
 //          range is split over many workgroups)
 //   Auto   Strip for layers of at least 128 tiles of 128 x 128 (2M weights), Full below
