@@ -45,6 +45,7 @@ struct BatchArgs {
     LutGeom geom;
     float lr_scale, rms_beta, rms_eps;
 };
+static_assert(sizeof(BatchArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
 // Per-workgroup tables in LDS (see counter_math.hpp).  fin and q_off depend on C only and are
 // built once per launch; c_reb depends on the row's scale ratio and is rebuilt per row.

@@ -79,6 +79,7 @@ struct GemmGroupArgs {
     GemmGroupItem it[kMaxGemmGroup];
     int n;
 };
+static_assert(sizeof(GemmGroupArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
 template <int BM, int BN>
 __global__ __launch_bounds__(kGemmThreads) void gemm_tn_group_kernel(GemmGroupArgs g) {
@@ -123,6 +124,7 @@ struct ReduceGroupArgs {
     ReduceGroupItem it[kMaxReduceGroup];
     int n;
 };
+static_assert(sizeof(ReduceGroupArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 constexpr int kReduceBlockElems = 256;  // one element per thread: a thread's chunk loads are all in flight at once
 
 __global__ __launch_bounds__(256) void reduce_slices_group_kernel(ReduceGroupArgs g) {
