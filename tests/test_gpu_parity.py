@@ -203,6 +203,25 @@ def test_matmul_transpose_a(ops, kmn):
     assert np.abs(c - ref).max() <= 1e-4 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("kmn", [(48, 4096, 4096), (32, 11008, 4096), (32, 4096, 11008)],
+                         ids=lambda s: "k%d_m%d_n%d" % s)
+def test_every_tile_shape_of_the_contraction_gives_the_same_bits(ops, kmn):
+    # 256 x 256 tiles, the row / column split with small tiles on the rest, and the 64 x 64 tiles a
+    # narrow block of the same operands gets: every output element sums its tokens in the same
+    # order, so the overlapping blocks must agree bit for bit
+    k, m, n = kmn
+    rng = np.random.default_rng(m + n)
+    a = rng.standard_normal((k, m)).astype(F)
+    b = rng.standard_normal((k, n)).astype(F)
+    full = host(ops.matmul_transpose_a(dev(a), dev(b)))
+    for r0 in (0, (m // 2) // 128 * 128, m - 128):
+        block = host(ops.matmul_transpose_a(dev(np.ascontiguousarray(a[:, r0:r0 + 128])), dev(b)))
+        assert np.array_equal(block, full[r0:r0 + 128]), r0
+    for c0 in (0, n - 128):
+        block = host(ops.matmul_transpose_a(dev(a), dev(np.ascontiguousarray(b[:, c0:c0 + 128]))))
+        assert np.array_equal(block, full[:, c0:c0 + 128]), c0
+
+
 FUSED_SHAPES = [  # (N, in, out, C)
     (2, 8, 2, 3),        # tests/test_vulkan_backend.cpp:1183
     (37, 68, 35, 3),     # tests/test_vulkan_counter_fused.cpp:57-60
