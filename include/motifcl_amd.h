@@ -138,7 +138,12 @@ void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
  *     calls must not run concurrently on one GPU (they could starve each
  *     other's waits), and mcc_compact_counter_fused_check reports a wait
  *     that was given up.
- * Both ways produce identical bytes.  grad_w differs from the reference's
+ * Both ways produce identical bytes whenever the first does not split the
+ * tokens into chunks, i.e. for fewer than 512 tokens or layers of at least
+ * 1024 tiles of 128 x 128 (mcc_compact_counter_fused_workspace_nbytes ==
+ * out*in*4); where it does, its gradient is the sum of chunk sums and the two
+ * ways differ by that rounding (a few counters in 10^5 flip differently).
+ * grad_w differs from the reference's
  * sequential fp32 sum only by summation order (relative error <= 1e-4 of the
  * row norm); given that grad_w the counter arithmetic is the same as in the
  * dense entry point.

@@ -20,7 +20,9 @@ namespace motifcl::nn {
 //          faster on large layers; the only way to keep the GPU busy on small ones, whose token
 //          range is split over many workgroups)
 //   Auto   Strip for layers of at least 128 tiles of 128 x 128 (2M weights), Full below
-// All give identical bytes.
+// Strip and Full give identical bytes wherever Full does not split the tokens into chunks (fewer
+// than 512 tokens, or at least 1024 tiles); elsewhere Full adds chunk sums and the two differ by
+// that rounding, both within the tolerance the contraction is held to.
 enum class FusedWorkspace { Auto, Strip, Full };
 
 class CounterStateLinear;
