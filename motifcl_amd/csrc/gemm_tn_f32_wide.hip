@@ -70,19 +70,31 @@ __global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_kernel(const flo
         if (k0 + kBK < k_len) issue(k0 + kBK, buf ^ 1);
         const float* lds_a = lds + buf * kWideSlabFloats;
         const float* lds_b = lds_a + kBK * kWide;
-#pragma unroll
-        for (int kk = 0; kk < kBK / 2; ++kk) {
-            float fa[4], fb[2];
+        // Operand reads run four steps ahead of the MFMAs that use them: while the next slab is
+        // being copied into LDS a read can take several times its usual latency, and with reads
+        // issued just in time the matrix pipe waits for them (one step ahead: 89.0 % of the peak on
+        // 4096 x 4096, two: 89.8 %, four: 90.3 %, six: 89.9 %).
+        constexpr int D = 4;
+        float fa[D + 1][4], fb[D + 1][2];
+        auto load = [&](int kk, int set) {
             const int krow = 2 * kk + half;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = lds_a[krow * kWide + wm0 + 32 * i + l32];
+            for (int i = 0; i < 4; ++i) fa[set][i] = lds_a[krow * kWide + wm0 + 32 * i + l32];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) fb[j] = lds_b[krow * kWide + wn0 + 32 * j + l32];
+            for (int j = 0; j < 2; ++j) fb[set][j] = lds_b[krow * kWide + wn0 + 32 * j + l32];
+        };
+#pragma unroll
+        for (int q = 0; q < D; ++q) load(q, q);
+#pragma unroll
+        for (int kk = 0; kk < kBK / 2; ++kk) {
+            if (kk + D < kBK / 2) load(kk + D, (kk + D) % (D + 1));
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[kk % (D + 1)][i], fb[kk % (D + 1)][j], acc[i][j], 0, 0, 0);
+            if (kk + D < kBK / 2) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
         }
         buf ^= 1;
     }
