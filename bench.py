@@ -37,8 +37,8 @@ BYTES_PER_PARAM = 5.5          # 4 (read G) + 0.75 (read state) + 0.75 (write st
 # 1 GiB copy; summaries and commands under profiles/).  They are reported, not re-measured
 # here, and only for the default workloads they were measured on.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg4/gemm_tn_f32": 8.91e9,       # average over the 7 contractions of a step (algorithmic 1.5 GB)
-    "cfg4/fused_strip": 27.43e9,      # average over the 7 launches of a step, --fused-path strip
+    "cfg4/gemm_tn_f32": 8.94e9,       # average over the 7 contractions of a step (algorithmic 1.5 GB)
+    "cfg4/fused_strip": 27.53e9,      # average over the 7 launches of a step, --fused-path strip
     "cfg3/update_rows": 36.16e9,      # the batched call of a step (algorithmic 35.64 GB)
 }
 
