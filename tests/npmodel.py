@@ -67,15 +67,22 @@ def row_stats(codes_row, g_row, scale_row, v_row, C, lr_scale, beta, eps):
     return vv, F(scale_new), F(denom)
 
 
-def tick(code, gw, s_old, s_new, dn, C, lr, seed, elem):
-    """One stochastic-rounding tick; the carry/remainder step is done on Python ints."""
+def draw_reference(seed, row, i, n_in):
+    """The draw of kernels/compact_counter.cl:121,127: the element index row*in + i is hashed,
+    xor-ed with the seed, and hashed again; the low 24 bits scale to [0, 1)."""
+    elem = (row * n_in + i) & 0xFFFFFFFF
+    return uniform01(seed ^ hash_u32(elem))
+
+
+def tick(code, gw, s_old, s_new, dn, C, lr, rnd):
+    """One stochastic-rounding tick for the draw `rnd`; the carry/remainder step is done on
+    Python ints."""
     lv = 2 * C - 1
     t, c = code // lv - 1, code % lv - (C - 1)
     Cf = F(C)
     tk = F(F(F(-F(lr)) * F(F(gw) / F(dn))) * F(Cf / F(s_new)))
     val = F(F(F(c) * F(F(s_old) / F(s_new))) + tk)
     f = np.floor(val)
-    rnd = uniform01(seed ^ hash_u32(elem))
     total = int(f) + (1 if rnd < F(val - f) else 0)     # integer-valued ccv
     carry = abs(total) // C * (1 if total >= 0 else -1)  # truncation toward zero
     rem = total - carry * C
@@ -87,7 +94,9 @@ def tick(code, gw, s_old, s_new, dn, C, lr, seed, elem):
     return (nt + 1) * lv + rem + (C - 1)
 
 
-def update_dense(state, scale, v, G, C, lr, lr_scale, beta, eps, seed):
+def update_dense(state, scale, v, G, C, lr, lr_scale, beta, eps, seed, draw=draw_reference):
+    """`draw(seed, row, i, n_in)` is the uniform variate of element (row, i); tests swap it to show
+    that a wrong composition of seed, index and hash does not reproduce the frozen vectors."""
     n_out, n_in = G.shape
     codes = unpack_state(state, n_out * n_in).reshape(n_out, n_in)
     new_codes = np.zeros_like(codes)
@@ -97,6 +106,6 @@ def update_dense(state, scale, v, G, C, lr, lr_scale, beta, eps, seed):
         vv, sn, dn = row_stats(codes[row], G[row], scale[row], v[row], C, lr_scale, beta, eps)
         for i in range(n_in):
             new_codes[row, i] = tick(int(codes[row, i]), G[row, i], scale[row], sn, dn, C, lr,
-                                     seed, (row * n_in + i) & 0xFFFFFFFF)
+                                     draw(seed, row, i, n_in))
         scale_out[row], v_out[row] = sn, vv
     return pack_state(new_codes), scale_out, v_out

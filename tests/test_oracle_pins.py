@@ -333,6 +333,94 @@ def test_draws_differ_across_elements_and_seeds(oracle):
     assert 1800 < ups < 2200
 
 
+# --------------------------------------------------------------------------- the draw's composition
+REF_COMP = "/root/reference/kernels/vulkan/counter_apply_update_fused_f32.comp"
+
+
+def _squash(text):
+    return re.sub(r"\s+", "", text)
+
+
+@pytest.mark.skipif(not (os.path.exists(REF_CL) and os.path.exists(REF_COMP)), reason="reference text not present")
+def test_draw_call_site_matches_reference_text():
+    # what the reference's three tick kernels write at the call site: the element index is
+    # row*in + 4g + k, hashed, xor-ed with the seed, and cc_uniform01 hashes the result again and
+    # keeps the LOW 24 bits.  Catches an oracle that follows a different reading of the text.
+    cl = open(REF_CL).read()
+    uni = _squash(cl[cl.index("cc_uniform01"):cl.index("cc_unpack4")])
+    assert "(float)(cc_hash_u32(x)&0x00ffffffu)*(1.0f/16777216.0f)" in uni
+    dense = _squash(cl[cl.index("void counter_apply_update_f32"):cl.index("void counter_row_stats_fused_f32")])
+    fused = _squash(cl[cl.index("void counter_apply_update_fused_f32"):])
+    draw = "floatrnd=cc_uniform01(seed^cc_hash_u32((uint)elem));"
+    assert dense.count(draw) == 1 and fused.count(draw) == 1
+    assert "intelem=row*in_features+g*4+k;" in dense
+    assert "inti=g*4+k;intelem=row*in_features+i;" in fused
+    for body in (dense, fused):
+        assert "introw=gid/gpr;intg=gid-row*gpr;" in body and "intgpr=in_features/4;" in body
+        assert "floatccv=f+(rnd<(val-f)?1.0f:0.0f);" in body
+    comp = _squash(open(REF_COMP).read())
+    assert "constfloatrnd=cc_uniform01(p.seed^cc_hash_u32(uint(elem)));" in comp
+    assert "constinti=g*4+k;constintelem=row*p.in_features+i;" in comp
+    assert "float(cc_hash_u32(h)&0x00ffffffu)*(1.0/16777216.0)" in comp
+
+
+def _u01_low24(x):
+    return npmodel.uniform01(x)
+
+
+def _u01_high24(x):
+    return F(npmodel.hash_u32(x) >> 8) * F(1.0 / 16777216.0)
+
+
+# plausible wrong readings of the call site: (name, draw(seed, row, i, n_in))
+_WRONG_DRAWS = [
+    ("index not hashed", lambda s, r, i, n: _u01_low24(s ^ ((r * n + i) & 0xFFFFFFFF))),
+    ("seed hashed instead of the index", lambda s, r, i, n: _u01_low24(npmodel.hash_u32(s) ^ ((r * n + i) & 0xFFFFFFFF))),
+    ("xor of two hashes", lambda s, r, i, n: _u01_low24(npmodel.hash_u32(s) ^ npmodel.hash_u32((r * n + i) & 0xFFFFFFFF))),
+    ("seed added, not xor-ed", lambda s, r, i, n: _u01_low24((s + npmodel.hash_u32((r * n + i) & 0xFFFFFFFF)) & 0xFFFFFFFF)),
+    ("no second hash", lambda s, r, i, n: F((s ^ npmodel.hash_u32((r * n + i) & 0xFFFFFFFF)) & 0xFFFFFF) * F(1.0 / 16777216.0)),
+    ("high 24 bits", lambda s, r, i, n: _u01_high24(s ^ npmodel.hash_u32((r * n + i) & 0xFFFFFFFF))),
+    ("row dropped from the index", lambda s, r, i, n: _u01_low24(s ^ npmodel.hash_u32(i))),
+    ("row stride in groups", lambda s, r, i, n: _u01_low24(s ^ npmodel.hash_u32((r * (n // 4) + i) & 0xFFFFFFFF))),
+    ("column-major index", lambda s, r, i, n: _u01_low24(s ^ npmodel.hash_u32((i * 35 + r) & 0xFFFFFFFF))),
+    ("group index instead of element index", lambda s, r, i, n: _u01_low24(s ^ npmodel.hash_u32((r * n + i) // 4))),
+    ("code position swapped inside the group", lambda s, r, i, n: _u01_low24(s ^ npmodel.hash_u32((r * n + (i ^ 3)) & 0xFFFFFFFF))),
+    ("one-based index", lambda s, r, i, n: _u01_low24(s ^ npmodel.hash_u32((r * n + i + 1) & 0xFFFFFFFF))),
+]
+
+
+def _frozen_case():
+    from tests import golden_cases as gc
+    dense, _ = gc.update_vectors()
+    c = dense[1]  # 35 x 68, C = 3: the shape of tests/test_vulkan_counter_fused.cpp:57-60
+    assert (c["n_out"], c["n_in"], c["C"]) == (35, 68, 3)
+    return c
+
+
+def _model_on(c, draw):
+    return npmodel.update_dense(c["state"], c["scale"], c["v"], c["G"], c["C"], c["lr"], c["lr_scale"],
+                                c["rms_beta"], c["rms_eps"], c["seed"], draw=draw)
+
+
+def test_frozen_vector_is_the_reference_draw():
+    # the committed vector is what the literal numpy model gives with the composition the
+    # reference text shows (test above) ...
+    c = _frozen_case()
+    st, sc, v = _model_on(c, npmodel.draw_reference)
+    assert np.array_equal(st, c["state_new"]) and np.array_equal(sc, c["scale_new"]) and np.array_equal(v, c["v_new"])
+
+
+@pytest.mark.parametrize("name,draw", _WRONG_DRAWS, ids=[n.replace(" ", "_") for n, _ in _WRONG_DRAWS])
+def test_frozen_vector_kills_wrong_draw_compositions(name, draw):
+    # ... and every plausible other composition lands hundreds of counters elsewhere, so an
+    # oracle or a kernel built on one of them cannot pass the frozen-vector tests
+    c = _frozen_case()
+    st, sc, v = _model_on(c, draw)
+    assert np.array_equal(sc, c["scale_new"]) and np.array_equal(v, c["v_new"])  # statistics do not use the draw
+    diff = (npmodel.unpack_state(st, 35 * 68) != npmodel.unpack_state(c["state_new"], 35 * 68)).sum()
+    assert diff >= 50, (name, diff)
+
+
 # --------------------------------------------------------------------------- whole update
 @pytest.mark.parametrize("shape", [(2, 8, 3), (5, 68, 3), (3, 264, 11), (2, 4, 1)])
 def test_update_dense_equals_numpy_model(oracle, shape):
