@@ -111,12 +111,6 @@ int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t 
                                     size_t in_features, size_t out_features, size_t batch);
 
 /*
- * Polls a strip-workspace step spends on one wait before giving up (0
- * restores the default, about four seconds).  For tests of the error path.
- */
-void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
-
-/*
  * Fused step: weight-gradient contraction grad_w = grad_out^T . x on the fp32
  * matrix cores followed by the counter update.
  * Replaces run_vulkan_compact_counter_apply_update_fused
@@ -322,19 +316,6 @@ int mcc_stream_synchronize(void* stream);
 void mcc_profiler_enable(int on);
 void mcc_profiler_reset(void);
 int mcc_profiler_query(const char* kernel_name, double* total_ms, uint64_t* launches);
-
-/*
- * Shader-clock probe (a measurement aid with no counterpart in the reference).
- * Enqueues a one-wave kernel on `stream` that sleeps for `seconds` (at most 2) of
- * the constant-rate wall clock and writes two 64-bit counts to the device buffer
- * `out`: out[0] wall-clock ticks, out[1] shader cycles over the same stretch.
- * Launched on a side stream while other kernels run it gives the frequency they
- * ran at: MHz = out[1] / out[0] * wall_clock_khz / 1000.  Matrix-core peaks are
- * quoted at the maximum engine clock; under load the power limit holds the clock
- * below it.
- */
-int mcc_clock_probe(void* stream, uint64_t* out, size_t out_nbytes, double seconds);
-int mcc_wall_clock_khz(int* khz);
 
 #ifdef __cplusplus
 }

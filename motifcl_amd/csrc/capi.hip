@@ -19,24 +19,30 @@
 #include "launch.hpp"
 
 namespace {
-
 thread_local std::string g_error;
+}  // namespace
 
-int fail(int code, const std::string& message) {
+namespace mcc {
+
+// Records the calling thread's failure message and returns `code` (shared with diag.hip).
+int report_failure(int code, const std::string& message) {
     g_error = message;
     return code;
 }
 
-int hip_fail(hipError_t e, const char* what) {
-    return fail(MCC_E_RUNTIME, std::string(what) + ": " + hipGetErrorString(e));
+int report_hip_failure(hipError_t e, const char* what) {
+    return report_failure(MCC_E_RUNTIME, std::string(what) + ": " + hipGetErrorString(e));
 }
 
-constexpr size_t kIntMax = static_cast<size_t>(std::numeric_limits<int>::max());
+}  // namespace mcc
 
-// Polls (about 0.25 us each) a strip-path workgroup spends on one wait before it gives up:
-// roughly four seconds, far above any wait a healthy launch can see.
-constexpr unsigned kDefaultStripSpinLimit = 1u << 24;
-std::atomic<unsigned> g_strip_spin_limit{kDefaultStripSpinLimit};
+namespace {
+
+int fail(int code, const std::string& message) { return mcc::report_failure(code, message); }
+
+int hip_fail(hipError_t e, const char* what) { return mcc::report_hip_failure(e, what); }
+
+constexpr size_t kIntMax = static_cast<size_t>(std::numeric_limits<int>::max());
 
 // 0: weight-gradient contraction on the fp32 matrix instruction; 1: split-bf16 form where the
 // shape allows it
@@ -245,10 +251,6 @@ size_t mcc_compact_counter_fused_strip_workspace_nbytes(size_t in_features, size
     return mcc::fused_strip_workspace_nbytes(in_features, out_features, batch);
 }
 
-void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins) {
-    g_strip_spin_limit.store(spins ? spins : kDefaultStripSpinLimit);
-}
-
 int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t workspace_nbytes,
                                     size_t in_features, size_t out_features, size_t batch) {
     if (!workspace) return fail(MCC_E_INVALID, "compact-counter fused check received a null workspace");
@@ -318,7 +320,7 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
         ScopedKernelTimer timer("fused_strip", s);
         e = mcc::launch_fused_strip(s, state, scale, v, grad_out, x, workspace, (int)C, (int)in_features,
                                     (int)out_features, (int)batch, lr, rms_beta, rms_eps, seed,
-                                    g_strip_spin_limit.load());
+                                    mcc::fused_strip_spin_limit());
         if (e != hipSuccess) return hip_fail(e, "compact-counter fused strip update launch failed");
         return MCC_OK;
     }
@@ -700,28 +702,6 @@ int mcc_memset_zero(void* stream, void* dst, size_t nbytes) {
                        static_cast<uint8_t*>(dst), nbytes);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e, "device memset failed");
-    return MCC_OK;
-}
-
-int mcc_wall_clock_khz(int* khz) {
-    if (!khz) return fail(MCC_E_INVALID, "wall_clock_khz received a null pointer");
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e == hipSuccess) e = hipDeviceGetAttribute(khz, hipDeviceAttributeWallClockRate, dev);
-    if (e != hipSuccess) return hip_fail(e, "wall_clock_khz query failed");
-    return MCC_OK;
-}
-
-int mcc_clock_probe(void* stream, uint64_t* out, size_t out_nbytes, double seconds) {
-    if (!out || out_nbytes < 2 * sizeof(uint64_t)) return fail(MCC_E_INVALID, "clock_probe needs a 16-byte device buffer");
-    if (!(seconds > 0.0) || seconds > 2.0) return fail(MCC_E_INVALID, "clock_probe duration must be in (0, 2] seconds");
-    int khz = 0;
-    const int rc = mcc_wall_clock_khz(&khz);
-    if (rc != MCC_OK) return rc;
-    const unsigned long long ticks = (unsigned long long)(seconds * 1e3 * (double)khz);
-    const hipError_t e =
-        mcc::launch_clock_probe(static_cast<hipStream_t>(stream), reinterpret_cast<unsigned long long*>(out), ticks);
-    if (e != hipSuccess) return hip_fail(e, "clock_probe launch failed");
     return MCC_OK;
 }
 

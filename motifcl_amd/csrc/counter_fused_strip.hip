@@ -29,6 +29,7 @@
 // ends all waits, and the host reports the failure.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 
 #include "counter_math.hpp"
@@ -381,6 +382,14 @@ constexpr size_t kHeaderBytes = 256;  // status word, padded
 size_t flags_bytes(size_t strips) { return (strips * 2 * sizeof(int) + 255) / 256 * 256; }
 
 }  // namespace
+
+// Polls (about 0.25 us each) a workgroup spends on one wait before it gives up: roughly four
+// seconds, far above any wait a healthy launch can see.
+constexpr unsigned kDefaultSpinLimit = 1u << 24;
+static std::atomic<unsigned> g_spin_limit{kDefaultSpinLimit};
+
+unsigned fused_strip_spin_limit() { return g_spin_limit.load(); }
+void set_fused_strip_spin_limit(unsigned spins) { g_spin_limit.store(spins ? spins : kDefaultSpinLimit); }
 
 bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch) {
     return batch > 0 && in_features >= kTile && out_features >= kTile && in_features % kTile == 0 &&

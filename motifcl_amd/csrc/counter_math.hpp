@@ -23,25 +23,36 @@ namespace mcc {
 // lowbias32 (kernels/compact_counter.cl:17-21), split after its first xor-shift: the four
 // elements of a packed group have indices e, e+1, e+2, e+3 with e a multiple of 4, and
 // (e + k) ^ ((e + k) >> 16) == (e ^ (e >> 16)) ^ k for k < 4, so the first step is shared.
+constexpr uint32_t kHashMul1 = 0x7feb352du, kHashMul2 = 0x846ca68bu;
+
 MCC_HD uint32_t hash_first(uint32_t x) { return x ^ (x >> 16); }
 
 MCC_HD uint32_t hash_rest(uint32_t x) {
-    x *= 0x7feb352du;
+    x *= kHashMul1;
     x ^= x >> 15;
-    x *= 0x846ca68bu;
+    x *= kHashMul2;
     x ^= x >> 16;
     return x;
 }
 
 MCC_HD uint32_t hash_u32(uint32_t x) { return hash_rest(hash_first(x)); }
 
-// hash_rest without its last xor-shift: hash_rest(x) == u ^ (u >> 16) with u = hash_open(x).
-MCC_HD uint32_t hash_open(uint32_t x) {
-    x *= 0x7feb352du;
-    x ^= x >> 15;
-    x *= 0x846ca68bu;
-    return x;
+// hash_rest without its last xor-shift, given its first product p = x * kHashMul1:
+// hash_rest(x) == u ^ (u >> 16) with u = hash_open_from_product(x * kHashMul1).
+MCC_HD uint32_t hash_open_from_product(uint32_t p) {
+    p ^= p >> 15;
+    p *= kHashMul2;
+    return p;
 }
+
+MCC_HD uint32_t hash_open(uint32_t x) { return hash_open_from_product(x * kHashMul1); }
+
+// The four elements of a group enter the inner hash as x ^ k, k = 0..3, with x = hash_first of
+// the group's first element.  x ^ k == x + ((s ^ k) - s) for s = x & 3, so their first products
+// are (x ^ k) * kHashMul1 == x * kHashMul1 + hash_delta(s, k) (mod 2^32): one multiplication and
+// three additions per group, and s -- bits 16..17 of the element index -- is the same for every
+// group of a 256-element aligned span.
+MCC_HD uint32_t hash_delta(uint32_t s, uint32_t k) { return ((s ^ k) - s) * kHashMul1; }
 
 // The draw of kernels/compact_counter.cl:127 is hash(seed ^ hash(elem)).  With h = u ^ (u >> 16)
 // the inner hash and y = seed ^ h, the outer hash starts with y ^ (y >> 16), and
@@ -51,8 +62,9 @@ MCC_HD uint32_t hash_open(uint32_t x) {
 // into one xor with a per-tensor constant.
 MCC_HD uint32_t seed_mix(uint32_t seed) { return seed ^ (seed >> 16); }
 
-// hash_u32(seed ^ hash_rest(x)) given mix = seed_mix(seed)
-MCC_HD uint32_t draw_hash(uint32_t mix, uint32_t x) { return hash_rest(mix ^ hash_open(x)); }
+// hash_u32(seed ^ hash_rest(x)) given mix = seed_mix(seed), from x or from p = x * kHashMul1
+MCC_HD uint32_t draw_hash_from_product(uint32_t mix, uint32_t p) { return hash_rest(mix ^ hash_open_from_product(p)); }
+MCC_HD uint32_t draw_hash(uint32_t mix, uint32_t x) { return draw_hash_from_product(mix, x * kHashMul1); }
 
 // 24-bit word of one packed group -> code k (kernels/compact_counter.cl:25-31)
 MCC_HD uint32_t code_of(uint32_t word, int k) { return (word >> (6 * k)) & 0x3fu; }
@@ -178,6 +190,16 @@ MCC_HD bool row_takes_fast_division(float dn, float row_sum_sq, uint32_t row_min
     return dn >= 0x1p-40f && dn <= 0x1p40f && row_sum_sq < 0x1p100f && row_min_key >= range_key(0x1p-60f);
 }
 
+// The same decision from the smallest |gw| of the row, zeros included (one v_min3_f32 per two
+// elements instead of a key per element): +1 fast, -1 exact division, 0 undecided -- the row
+// holds an exact zero, which hides whether it also holds a non-zero value below 2^-60, and the
+// caller looks again with range_key.
+MCC_HD int fast_division_from_min_abs(float dn, float row_sum_sq, float row_min_abs) {
+    if (!(dn >= 0x1p-40f && dn <= 0x1p40f && row_sum_sq < 0x1p100f)) return -1;
+    if (row_min_abs >= 0x1p-60f) return 1;
+    return row_min_abs == 0.0f ? 0 : -1;
+}
+
 template <bool FAST>
 MCC_HD float div_by_row(float gw, float dn, float r) {
     if (!FAST) return gw / dn;
@@ -212,18 +234,25 @@ struct TickConsts {
 //   elem_x : hash_first(row*in + i), the RNG index after the first xor-shift
 //   c_reb, q_off : the decode tables above;  fin : the (q, total) -> code table
 // Returns the new 6-bit code.
+//   first_product : hash_first(row*in + i) * kHashMul1 (see hash_delta)
 template <bool FAST_DIV, typename CReb, typename QOff, typename Fin>
-MCC_HD uint32_t tick_code(uint32_t code, float gw, const TickConsts& tc, uint32_t elem_x,
-                          CReb c_reb, QOff q_off, Fin fin) {
+MCC_HD uint32_t tick_code_from_product(uint32_t code, float gw, const TickConsts& tc, uint32_t first_product,
+                                       CReb c_reb, QOff q_off, Fin fin) {
     const float tick = (tc.neg_lr * div_by_row<FAST_DIV>(gw, tc.dn, tc.r)) * tc.k;
     const float val = c_reb[code] + tick;
     const float f = floorf(val);
     const float frac = val - f;
-    const uint32_t h = draw_hash(tc.seed_mix, elem_x);
+    const uint32_t h = draw_hash_from_product(tc.seed_mix, first_product);
     const float rnd = (float)(h & 0x00ffffffu) * tc.two_m24;
     // q_off + floor + [rnd < frac]: one add-with-carry on the GPU
     const int idx = q_off[code] + (int)clamp_f(f, tc.neg_lim_neg, tc.lim_pos) + (rnd < frac ? 1 : 0);
     return fin[idx];
+}
+
+template <bool FAST_DIV, typename CReb, typename QOff, typename Fin>
+MCC_HD uint32_t tick_code(uint32_t code, float gw, const TickConsts& tc, uint32_t elem_x,
+                          CReb c_reb, QOff q_off, Fin fin) {
+    return tick_code_from_product<FAST_DIV>(code, gw, tc, elem_x * kHashMul1, c_reb, q_off, fin);
 }
 
 // Row statistics epilogue (kernels/compact_counter.cl:92-99), given the tree

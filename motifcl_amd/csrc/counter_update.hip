@@ -34,8 +34,7 @@ namespace mcc {
 namespace {
 
 constexpr int kWave = 64;
-constexpr int kWavesPerBlock = 1;  // one wave per workgroup: the row index is a function of blockIdx alone
-constexpr int kThreads = kWave * kWavesPerBlock;
+constexpr int kThreads = kWave;  // one wave per workgroup: the row index is a function of blockIdx alone
 
 struct BatchArgs {
     UpdateTensor t[kMaxUpdateBatch];
@@ -84,10 +83,21 @@ __device__ __forceinline__ uint32_t load_group_dword(const uint8_t* p) {
     return w;
 }
 
-// Row statistics of one group (kernels/compact_counter.cl:78-83) plus the magnitude key
-// that decides whether the row may use the reciprocal-based division.
+// The same for a group that may be the tensor's last (`tail`): that one has no byte after it, so
+// it is fetched one byte early and shifted down.  The tensor holds at least two groups (the
+// launch sends smaller ones to the byte-granular kernel), so the byte before exists.
+__device__ __forceinline__ uint32_t load_group_dword_or_tail(const uint8_t* p, bool tail) {
+    const uint32_t back = tail ? 1u : 0u;
+    return load_group_dword(p - back) >> (8u * back);
+}
+
+// Row statistics of one group (kernels/compact_counter.cl:78-83) plus what decides whether the
+// row may use the reciprocal-based division: the smallest |g| of the row (zeros included, one
+// v_min3_f32 per two elements) in the register-resident kernels, the exact magnitude key (zero
+// mapped above everything) in the streamed ones.
 struct RowAcc {
     float g_sq = 0.0f, grad_s = 0.0f;
+    float min_abs = __builtin_inff();
     uint32_t min_key = 0xffffffffu;
 };
 
@@ -96,10 +106,27 @@ __device__ __forceinline__ uint32_t umin3(uint32_t a, uint32_t b, uint32_t c) {
     return c < ab ? c : ab;  // one v_min3_u32
 }
 
-template <bool WITH_GS>
-__device__ __forceinline__ void accumulate(RowAcc& acc, const float g[4], uint32_t w, const Codec& cd) {
-    acc.min_key = umin3(acc.min_key, range_key(g[0]), range_key(g[1]));
-    acc.min_key = umin3(acc.min_key, range_key(g[2]), range_key(g[3]));
+__device__ __forceinline__ float fmin3_abs(float a, float b, float c) {
+    return __builtin_fminf(__builtin_fminf(a, __builtin_fabsf(b)), __builtin_fabsf(c));  // one v_min3_f32 with |.| modifiers
+}
+
+// Smallest magnitude key of one group (zero counts as large).
+__device__ __forceinline__ uint32_t group_min_key(uint32_t key, const float g[4]) {
+    key = umin3(key, range_key(g[0]), range_key(g[1]));
+    return umin3(key, range_key(g[2]), range_key(g[3]));
+}
+
+// `g` holds zeros for a group past the end of the row (they add +0.0 to the squares and -+0.0 to
+// the products with t, which leaves both sums unchanged); `live` keeps such a group out of the
+// minimum as well.
+template <bool WITH_GS, bool EXACT_KEY>
+__device__ __forceinline__ void accumulate(RowAcc& acc, const float g[4], bool live, uint32_t w, const Codec& cd) {
+    if (EXACT_KEY) {
+        acc.min_key = group_min_key(acc.min_key, g);
+    } else {
+        const float m = fmin3_abs(fmin3_abs(acc.min_abs, g[0], g[1]), g[2], g[3]);
+        acc.min_abs = live ? m : acc.min_abs;
+    }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const float sq = g[k] * g[k];
@@ -125,22 +152,34 @@ __device__ __forceinline__ uint32_t wave_min(uint32_t a, int lane) {
     return (uint32_t)__builtin_amdgcn_readfirstlane((int)a);
 }
 
+// Non-negative floats order like their bit patterns.
+__device__ __forceinline__ float wave_min_nonneg(float a, int lane) { return __uint_as_float(wave_min(__float_as_uint(a), lane)); }
+
 struct RowCtx {
     TickConsts tc;
     bool fast_div;  // wave-uniform
 };
 
-// Tree reduction, row epilogue, commit of v/scale, and the per-row c_reb table.
-template <bool WITH_GS>
+// Tree reduction, row epilogue, commit of v/scale, and the per-row c_reb table.  `exact_key()`
+// returns the lane's exact magnitude key over the row; it is called (by the whole wave) only when
+// the smallest magnitude cannot decide, i.e. when the row holds an exact zero.
+template <bool WITH_GS, bool EXACT_KEY, typename KeyFn>
 __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTensor& t, int row, int lane,
-                                             const RowAcc& acc, Luts& l) {
+                                             const RowAcc& acc, Luts& l, KeyFn exact_key) {
     const float g_sq = tree_sum(acc.g_sq, lane);
     const float grad_s = WITH_GS ? tree_sum(acc.grad_s, lane) : 0.0f;
-    const uint32_t min_key = wave_min(acc.min_key, lane);
     const float s_old = t.scale[row];
     const float v_old = t.v[row];
     const RowStats rs = finish_row_stats(g_sq, grad_s, v_old, s_old, t.in_features, a.lr_scale,
                                          a.rms_beta, a.rms_eps);
+    int fast;
+    if (EXACT_KEY) {
+        fast = row_takes_fast_division(rs.denom, g_sq, wave_min(acc.min_key, lane)) ? 1 : -1;
+    } else {
+        fast = fast_division_from_min_abs(rs.denom, g_sq, wave_min_nonneg(acc.min_abs, lane));
+        fast = __builtin_amdgcn_readfirstlane(fast);
+        if (fast == 0) fast = row_takes_fast_division(rs.denom, g_sq, wave_min(exact_key(), lane)) ? 1 : -1;
+    }
     if (lane == 0) {
         t.v[row] = rs.v_new;
         t.scale[row] = rs.scale_new;  // commit (kernels/basic.cl:6-9); s_old stays in a register
@@ -157,12 +196,14 @@ __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTen
     rc.tc.lim_pos = (float)a.geom.lim_pos;
     rc.tc.seed_mix = seed_mix(t.seed);
     rc.tc.two_m24 = 1.0f / 16777216.0f;
-    // v_mul_f32 issues at twice the rate when both operands are VGPRs: keep the per-row
-    // multipliers out of scalar registers and literals
-    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24));
-    rc.fast_div = __builtin_amdgcn_readfirstlane(row_takes_fast_division(rs.denom, g_sq, min_key) ? 1 : 0) != 0;
+    // two-register VOP2 forms issue faster than forms with a scalar or literal operand: keep the
+    // per-row operands of the per-element instructions in vector registers
+    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24), "+v"(rc.tc.seed_mix));
+    rc.fast_div = __builtin_amdgcn_readfirstlane(fast > 0 ? 1 : 0) != 0;
     return rc;
 }
+
+__device__ __forceinline__ uint32_t no_exact_key() { return 0xffffffffu; }
 
 template <bool FAST_DIV>
 __device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], const TickConsts& tc,
@@ -172,6 +213,21 @@ __device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], con
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const uint32_t nc = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, x0 ^ (uint32_t)k, l.c_reb, l.q_off, l.fin);
+        nw |= nc << (6 * k);
+    }
+    return nw;
+}
+
+// The same for a group whose first products come by addition (hash_delta): p0 is
+// hash_first(elem0) * kHashMul1 and d[k-1] the wave-uniform delta of element k.
+template <bool FAST_DIV>
+__device__ __forceinline__ uint32_t tick_group_deltas(uint32_t w, const float g[4], const TickConsts& tc,
+                                                      const Luts& l, uint32_t p0, const uint32_t d[3]) {
+    uint32_t nw = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t p = k == 0 ? p0 : p0 + d[k - 1];
+        const uint32_t nc = tick_code_from_product<FAST_DIV>(code_of(w, k), g[k], tc, p, l.c_reb, l.q_off, l.fin);
         nw |= nc << (6 * k);
     }
     return nw;
@@ -195,47 +251,67 @@ __device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, i
     }
 }
 
-// One row, held in registers: ITERS == ceil(gpr / 64) exactly, grad_w 16-byte aligned, and the
-// row is not the last of its tensor (so reading one byte past any of its groups stays inside
-// the state).  Every iteration but the last covers 64 full groups, so its loads, sums and
-// stores need no masks and all addresses are one per-lane base plus a compile-time offset;
-// in the last iteration lanes past the end of the row re-read the row's last group and are
-// masked out of the sums and of the store.  All loads are issued back to back.
-template <int ITERS, bool WITH_GS>
-__device__ __forceinline__ void update_row_resident(const BatchArgs& a, const UpdateTensor& t, int row,
-                                                    int lane, Luts& luts) {
-    constexpr bool kKeepWords = ITERS <= 16;  // longer rows re-read their state words (cache hits)
+// A row held in registers: ITERS == ceil(gpr / 64) exactly and grad_w 16-byte aligned.  State words
+// are fetched with 4-byte loads that reach one byte past their group.
+// Every iteration but the last covers 64 full groups, so its loads, sums and stores need no masks
+// and all addresses are one per-lane base plus a compile-time offset; in the last iteration lanes
+// past the end of the row re-read the row's last group and are masked out of the sums and of the
+// store.  EXACT: the row is exactly 256 * ITERS weights, no lane is ever masked, and every
+// iteration's 256 elements are an aligned span of the element index, so the first products of
+// the inner hash come by addition (hash_delta).
+template <int ITERS, bool EXACT>
+__device__ __forceinline__ void load_row(const UpdateTensor& t, int row, int lane, float4 (&q)[ITERS],
+                                         uint32_t (&w)[ITERS]) {
     constexpr int kLast = ITERS - 1;
     const uint32_t gpr = (uint32_t)t.in_features >> 2;
     const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
-    uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    const uint8_t* s_row = t.state + (size_t)row * gpr * 3;
     const uint32_t gi_last = (uint32_t)lane + kWave * kLast;
-    const bool last_live = gi_last < gpr;
-    const uint32_t gc_last = last_live ? gi_last : gpr - 1;
-
-    float4 q[ITERS];
-    uint32_t w[kKeepWords ? ITERS : 1];
+    const uint32_t gc_last = EXACT || gi_last < gpr ? gi_last : gpr - 1;
+    const bool last_row = row == t.out_features - 1;  // wave-uniform
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const uint32_t gc = j < kLast ? (uint32_t)lane + kWave * j : gc_last;
         q[j] = g_row[gc];
-        if (kKeepWords) w[j] = load_group_dword(s_row + 3u * gc);
+        // only the row's last iteration can hold the tensor's last group
+        w[j] = j < kLast ? load_group_dword(s_row + 3u * gc)
+                         : load_group_dword_or_tail(s_row + 3u * gc, last_row && gc == gpr - 1);
     }
+}
+
+// One register-resident row: all loads are issued back to back (one contiguous burst per row,
+// which is also what the memory likes best: fetching the next row piecemeal during this row's
+// ticks was measured 10-30 % slower), then statistics, row epilogue and ticks.
+template <int ITERS, bool WITH_GS, bool EXACT>
+__device__ __forceinline__ void update_row_resident(const BatchArgs& a, const UpdateTensor& t, int row, int lane,
+                                                    Luts& luts) {
+    constexpr int kLast = ITERS - 1;
+    const uint32_t gpr = (uint32_t)t.in_features >> 2;
+    uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    const bool last_live = EXACT || (uint32_t)lane + kWave * kLast < gpr;
+    float4 q[ITERS];
+    uint32_t w[ITERS];
+    load_row<ITERS, EXACT>(t, row, lane, q, w);
+
     RowAcc acc;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const bool live = j < kLast || last_live;
-        // a masked group adds +0.0 (squares) and -+0.0 (0 * t): both leave the sums unchanged
         const float g[4] = {live ? q[j].x : 0.0f, live ? q[j].y : 0.0f, live ? q[j].z : 0.0f,
                             live ? q[j].w : 0.0f};
-        uint32_t word = 0;
-        if (WITH_GS) {
-            const uint32_t gc = j < kLast ? (uint32_t)lane + kWave * j : gc_last;
-            word = kKeepWords ? w[j] : load_group_dword(s_row + 3u * gc);
-        }
-        accumulate<WITH_GS>(acc, g, word, a.cd);
+        accumulate<WITH_GS, false>(acc, g, live, w[j], a.cd);
     }
-    const RowCtx rc = finish_row<WITH_GS>(a, t, row, lane, acc, luts);
+    const RowCtx rc = finish_row<WITH_GS, false>(a, t, row, lane, acc, luts, [&]() {
+        uint32_t key = 0xffffffffu;
+#pragma unroll
+        for (int j = 0; j < ITERS; ++j) {
+            const bool live = j < kLast || last_live;
+            const float g[4] = {live ? q[j].x : 0.0f, live ? q[j].y : 0.0f, live ? q[j].z : 0.0f,
+                                live ? q[j].w : 0.0f};
+            key = group_min_key(key, g);
+        }
+        return key;
+    });
     if (!rc.fast_div) {
         apply_streamed(t, row, lane, rc.tc, luts);
         return;
@@ -244,10 +320,17 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const uint32_t gi = (uint32_t)lane + kWave * j;
-        const uint32_t gc = j < kLast ? gi : gc_last;
         const float g[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
-        const uint32_t word = kKeepWords ? w[j] : load_group_dword(s_row + 3u * gc);
-        const uint32_t nw = tick_group<true>(word, g, rc.tc, luts, row_elem + 4u * gi);
+        uint32_t nw;
+        if (EXACT) {
+            // wave-uniform: bits 16..17 of the element index are the same over this aligned span
+            const uint32_t span = row_elem + 4u * kWave * j;
+            const uint32_t sbits = (span >> 16) & 3u;
+            const uint32_t d[3] = {hash_delta(sbits, 1), hash_delta(sbits, 2), hash_delta(sbits, 3)};
+            nw = tick_group_deltas<true>(w[j], g, rc.tc, luts, hash_first(span + 4u * (uint32_t)lane) * kHashMul1, d);
+        } else {
+            nw = tick_group<true>(w[j], g, rc.tc, luts, row_elem + 4u * gi);
+        }
         if (j < kLast || last_live) store_group(s_row + 3u * gi, nw);
     }
 }
@@ -264,13 +347,20 @@ __device__ __forceinline__ void update_row_streamed(const BatchArgs& a, const Up
         float g[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) g[k] = g_row[4 * gi + k];
-        accumulate<WITH_GS>(acc, g, load_group(s_row + 3 * gi), a.cd);
+        accumulate<WITH_GS, true>(acc, g, true, load_group(s_row + 3 * gi), a.cd);
     }
-    const RowCtx rc = finish_row<WITH_GS>(a, t, row, lane, acc, luts);
+    const RowCtx rc = finish_row<WITH_GS, true>(a, t, row, lane, acc, luts, no_exact_key);
     apply_streamed(t, row, lane, rc.tc, luts);
 }
 
-// One row of any length, 16-byte aligned, not the last of its tensor, by one wave in two passes
+// State word of group gc of a row; `last_row` (wave-uniform) tells that the row is the tensor's
+// last, whose final group needs the early fetch.
+__device__ __forceinline__ uint32_t load_row_word(const uint8_t* s_row, uint32_t gc, uint32_t gpr, bool last_row) {
+    if (last_row) return load_group_dword_or_tail(s_row + 3u * gc, gc == gpr - 1);
+    return load_group_dword(s_row + 3u * gc);
+}
+
+// One row of any length, 16-byte aligned, by one wave in two passes
 // over the row: statistics first, ticks second.  The second pass finds the row in L2 or in the
 // memory-side cache as long as the rows in flight fit there (5 waves per SIMD: 5120 rows, i.e.
 // 100-230 MB at 5120-11008 weights a row); what the two passes buy is a register footprint of
@@ -286,6 +376,7 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
     const int iters = (int)((gpr + kWave - 1) / kWave);
     const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    const bool last_row = row == t.out_features - 1;
     RowAcc acc;
     for (int c0 = 0; c0 < iters; c0 += kChunk) {
         float4 q[kChunk];
@@ -295,7 +386,7 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
             const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j);
             const uint32_t gc = gi < gpr ? gi : gpr - 1;
             q[j] = g_row[gc];
-            if (WITH_GS) w[j] = load_group_dword(s_row + 3u * gc);
+            if (WITH_GS) w[j] = load_row_word(s_row, gc, gpr, last_row);
         }
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) {
@@ -303,10 +394,10 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
             const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j) < gpr;
             const float g[4] = {live ? q[j].x : 0.0f, live ? q[j].y : 0.0f, live ? q[j].z : 0.0f,
                                 live ? q[j].w : 0.0f};
-            accumulate<WITH_GS>(acc, g, WITH_GS ? w[j] : 0u, a.cd);
+            accumulate<WITH_GS, true>(acc, g, live, WITH_GS ? w[j] : 0u, a.cd);
         }
     }
-    const RowCtx rc = finish_row<WITH_GS>(a, t, row, lane, acc, luts);
+    const RowCtx rc = finish_row<WITH_GS, true>(a, t, row, lane, acc, luts, no_exact_key);
     if (!rc.fast_div) {
         apply_streamed(t, row, lane, rc.tc, luts);
         return;
@@ -320,7 +411,7 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
             const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j);
             const uint32_t gc = gi < gpr ? gi : gpr - 1;
             q[j] = g_row[gc];
-            w[j] = load_group_dword(s_row + 3u * gc);
+            w[j] = load_row_word(s_row, gc, gpr, last_row);
         }
 #pragma unroll
         for (int j = 0; j < kChunk; ++j) {
@@ -337,35 +428,41 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
 // Minimum waves per SIMD the compiler must leave room for: the tick arithmetic has long
 // dependent chains, so the row's registers are budgeted to keep 3-4 waves resident for short
 // rows and 2 for the longest.
-#ifndef MCC_MIN_WAVES_16
-#define MCC_MIN_WAVES_16 3
-#endif
-constexpr int min_waves(int iters) { return iters <= 10 ? 4 : (iters <= 16 ? MCC_MIN_WAVES_16 : 2); }
+constexpr int min_waves(int iters) { return iters <= 10 ? 4 : (iters <= 16 ? 3 : 2); }
 
-template <int ITERS, bool WITH_GS>
+// The tensor that holds row `grow` of the launch's concatenated row space; ti only moves forward.
+// Everything here depends on blockIdx and kernel arguments only, so it lives in scalar registers.
+__device__ __forceinline__ UpdateTensor locate_row(const BatchArgs& a, int grow, int& ti) {
+    ti = __builtin_amdgcn_readfirstlane(ti);
+    while (grow >= a.t[ti].row_start + a.t[ti].out_features) ++ti;  // monotonic
+    ti = __builtin_amdgcn_readfirstlane(ti);
+    return a.t[ti];
+}
+
+template <int ITERS, bool WITH_GS, bool EXACT>
 __global__ __launch_bounds__(kThreads, min_waves(ITERS)) void update_rows_kernel(BatchArgs a) {
     __shared__ Luts luts;
     build_luts(luts, a.cd, a.geom);
     const int lane = threadIdx.x;
-    // everything that selects the row depends on blockIdx only, so it lives in scalar registers
-    const int wave = blockIdx.x;
-    const int stride = gridDim.x;
     int ti = 0;
-    for (int grow_v = wave; grow_v < a.total_rows; grow_v += stride) {
-        // readfirstlane pins the row and tensor index into scalar registers, so the descriptor
-        // fields below are scalar loads from the kernel-argument segment
+    for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
         const int grow = __builtin_amdgcn_readfirstlane(grow_v);
-        ti = __builtin_amdgcn_readfirstlane(ti);
-        while (grow >= a.t[ti].row_start + a.t[ti].out_features) ++ti;  // monotonic
-        ti = __builtin_amdgcn_readfirstlane(ti);
-        const UpdateTensor t = a.t[ti];
-        const int row = grow - t.row_start;
-        // the tensor's last row goes through the byte-granular path: its last group has no
-        // byte after it for the 4-byte state load
-        if (ITERS > 0 && row != t.out_features - 1)
-            update_row_resident<(ITERS > 0 ? ITERS : 1), WITH_GS>(a, t, row, lane, luts);
-        else
-            update_row_streamed<WITH_GS>(a, t, row, lane, luts);
+        const UpdateTensor t = locate_row(a, grow, ti);
+        update_row_resident<ITERS, WITH_GS, EXACT>(a, t, grow - t.row_start, lane, luts);
+    }
+}
+
+// Rows of any length and alignment, streamed (read twice).
+template <bool WITH_GS>
+__global__ __launch_bounds__(kThreads, 4) void update_rows_streamed_kernel(BatchArgs a) {
+    __shared__ Luts luts;
+    build_luts(luts, a.cd, a.geom);
+    const int lane = threadIdx.x;
+    int ti = 0;
+    for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
+        const int grow = __builtin_amdgcn_readfirstlane(grow_v);
+        const UpdateTensor t = locate_row(a, grow, ti);
+        update_row_streamed<WITH_GS>(a, t, grow - t.row_start, lane, luts);
     }
 }
 
@@ -377,15 +474,8 @@ __global__ __launch_bounds__(kThreads, 4) void update_rows_long_kernel(BatchArgs
     int ti = 0;
     for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
         const int grow = __builtin_amdgcn_readfirstlane(grow_v);
-        ti = __builtin_amdgcn_readfirstlane(ti);
-        while (grow >= a.t[ti].row_start + a.t[ti].out_features) ++ti;  // monotonic
-        ti = __builtin_amdgcn_readfirstlane(ti);
-        const UpdateTensor t = a.t[ti];
-        const int row = grow - t.row_start;
-        if (row != t.out_features - 1)
-            update_row_two_pass<WITH_GS>(a, t, row, lane, luts);
-        else
-            update_row_streamed<WITH_GS>(a, t, row, lane, luts);
+        const UpdateTensor t = locate_row(a, grow, ti);
+        update_row_two_pass<WITH_GS>(a, t, grow - t.row_start, lane, luts);
     }
 }
 
@@ -417,22 +507,9 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
     int ti = 0;
     for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
         const int grow = __builtin_amdgcn_readfirstlane(grow_v);
-        ti = __builtin_amdgcn_readfirstlane(ti);
-        while (grow >= a.t[ti].row_start + a.t[ti].out_features) ++ti;  // monotonic
-        ti = __builtin_amdgcn_readfirstlane(ti);
-        const UpdateTensor t = a.t[ti];
+        const UpdateTensor t = locate_row(a, grow, ti);
         const int row = grow - t.row_start;
-        if (row == t.out_features - 1) {
-            // byte-granular path for the tensor's last row, by wave 0; the others only keep the
-            // workgroup's barrier count in step (finish_row synchronises twice)
-            if (w == 0) {
-                update_row_streamed<WITH_GS>(a, t, row, lane, sh.luts);
-            } else {
-                __syncthreads();
-                __syncthreads();
-            }
-            continue;
-        }
+        const bool last_row = row == t.out_features - 1;
         const uint32_t gpr = (uint32_t)t.in_features >> 2;
         const int iters = (int)((gpr + kWave - 1) / kWave);
         const int j0 = w * J;
@@ -446,7 +523,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
             const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
             const uint32_t gc = gi < gpr ? gi : gpr - 1;
             q[jj] = g_row[gc];
-            words[jj] = load_group_dword(s_row + 3u * gc);
+            words[jj] = load_row_word(s_row, gc, gpr, last_row);
         }
         // What does not depend on the order happens before the hand-off, in all waves at once: the
         // squares, the products with t, and the minimum of the magnitude keys (a minimum may be
@@ -494,7 +571,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
                         const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
                         const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
                                             live ? q[jj].w : 0.0f};
-                        accumulate<WITH_GS>(acc, g, words[jj], a.cd);
+                        accumulate<WITH_GS, true>(acc, g, live, words[jj], a.cd);
                     }
                 }
                 if (step < W - 1) {
@@ -561,19 +638,33 @@ int device_cu_count() {
     return cus;
 }
 
-template <int ITERS, bool WITH_GS>
+template <int ITERS, bool WITH_GS, bool EXACT>
 hipError_t launch_variant(hipStream_t stream, const BatchArgs& a) {
     static int blocks_per_cu = [] {
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_kernel<ITERS, WITH_GS>, kThreads, 0) != hipSuccess ||
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_kernel<ITERS, WITH_GS, EXACT>, kThreads, 0) !=
+                hipSuccess || n <= 0)
+            n = 2;
+        return n;
+    }();
+    const int resident = device_cu_count() * blocks_per_cu;
+    const dim3 grid(a.total_rows < resident ? a.total_rows : resident);
+    hipLaunchKernelGGL((update_rows_kernel<ITERS, WITH_GS, EXACT>), grid, dim3(kThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <bool WITH_GS>
+hipError_t launch_streamed_variant(hipStream_t stream, const BatchArgs& a) {
+    static int blocks_per_cu = [] {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_streamed_kernel<WITH_GS>, kThreads, 0) != hipSuccess ||
             n <= 0)
             n = 2;
         return n;
     }();
-    const int want = (a.total_rows + kWavesPerBlock - 1) / kWavesPerBlock;
     const int resident = device_cu_count() * blocks_per_cu;
-    const dim3 grid(want < resident ? want : resident);
-    hipLaunchKernelGGL((update_rows_kernel<ITERS, WITH_GS>), grid, dim3(kThreads), 0, stream, a);
+    const dim3 grid(a.total_rows < resident ? a.total_rows : resident);
+    hipLaunchKernelGGL(update_rows_streamed_kernel<WITH_GS>, grid, dim3(kThreads), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -614,34 +705,33 @@ hipError_t launch_split(hipStream_t stream, const BatchArgs& a) {
     return a.lr_scale != 0.0f ? launch_split_variant<J, W, true>(stream, a) : launch_split_variant<J, W, false>(stream, a);
 }
 
-template <int ITERS>
+template <int ITERS, bool EXACT>
 hipError_t launch_iters(hipStream_t stream, const BatchArgs& a) {
-    return a.lr_scale != 0.0f ? launch_variant<ITERS, true>(stream, a) : launch_variant<ITERS, false>(stream, a);
+    return a.lr_scale != 0.0f ? launch_variant<ITERS, true, EXACT>(stream, a) : launch_variant<ITERS, false, EXACT>(stream, a);
 }
 
 // Row lengths (in units of 64 groups = 256 weights, rounded up) with a one-wave
 // register-resident variant: every length up to 4096 weights.  Longer rows are read twice by
 // one wave, except 8192 < length <= 11264, which four waves share register-resident.
-#ifdef MCC_EXPERIMENT_FEW_VARIANTS
-#define MCC_RESIDENT_ITERS(X) X(3) X(8) X(16)
-#else
 #define MCC_RESIDENT_ITERS(X) \
     X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16)
-#endif
 
-// Classes of the split kernel are encoded as 1000 + 10*J + W.
+// Classes of the split kernel are encoded as 1000 + 10*J + W; a register-resident class is the
+// row's iteration count, plus kExactClass when the row is exactly 256 weights per iteration.
 constexpr int split_class(int j, int w) { return 1000 + 10 * j + w; }
+constexpr int kExactClass = 100;
 
 // Register-resident variant of a row of `in_features` (0 = streamed fallback).
 int iters_class(const UpdateTensor& t) {
     const int iters = ((t.in_features >> 2) + kWave - 1) / kWave;
     const bool aligned = (reinterpret_cast<uintptr_t>(t.grad_w) & 15u) == 0;
-    if (!aligned) return 0;
+    // a one-group tensor has no byte before its last group for the early fetch of that group
+    if (!aligned || (long)t.out_features * (t.in_features >> 2) < 2) return 0;
     switch (iters) {
 #define MCC_CASE(N) case N:
         MCC_RESIDENT_ITERS(MCC_CASE)
 #undef MCC_CASE
-        return iters;
+        return iters + (t.in_features == 4 * kWave * iters ? kExactClass : 0);
         default: break;
     }
     // 11008-wide rows (the 7B FFN width) stay with four cooperating waves, which read the row
@@ -655,13 +745,16 @@ int iters_class(const UpdateTensor& t) {
 
 hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
     switch (cls) {
-#define MCC_CASE(N) case N: return launch_iters<N>(stream, a);
+#define MCC_CASE(N)                                  \
+    case N: return launch_iters<N, false>(stream, a); \
+    case N + kExactClass: return launch_iters<N, true>(stream, a);
         MCC_RESIDENT_ITERS(MCC_CASE)
 #undef MCC_CASE
         case kLongClass:
             return a.lr_scale != 0.0f ? launch_long_variant<true>(stream, a) : launch_long_variant<false>(stream, a);
         case split_class(11, 4): return launch_split<11, 4>(stream, a);
-        default: return launch_iters<0>(stream, a);
+        default:
+            return a.lr_scale != 0.0f ? launch_streamed_variant<true>(stream, a) : launch_streamed_variant<false>(stream, a);
     }
 }
 

@@ -5,8 +5,13 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <string>
 
 namespace mcc {
+
+// Failure reporting of the C ABI (capi.hip): stores the message mcc_last_error() returns.
+int report_failure(int code, const std::string& message);
+int report_hip_failure(hipError_t e, const char* what);
 
 // One counter tensor of an update-only batch (device pointers).
 struct UpdateTensor {
@@ -67,6 +72,10 @@ hipError_t launch_gemm_tn_bf16x6(hipStream_t stream, const float* a, const float
 // Shapes: in_features and out_features multiples of 128; lr_scale == 0 is implied.
 bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch);
 size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch);
+// Polls one device-side wait of the strip step may spend before it gives up (0 restores the
+// default, about four seconds; a test aid declared in motifcl_amd_diag.h).
+unsigned fused_strip_spin_limit();
+void set_fused_strip_spin_limit(unsigned spins);
 hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, float* v,
                               const float* grad_out, const float* x, void* workspace, int C,
                               int in_features, int out_features, int tokens, float lr, float rms_beta,
@@ -90,8 +99,5 @@ hipError_t launch_sgd_update(hipStream_t stream, float* param, const float* grad
 hipError_t launch_adam_update(hipStream_t stream, float* param, const float* grad, float* m, float* v,
                               size_t n, float lr, float beta1, float beta2, float eps, float inv_bias1,
                               float inv_bias2, float weight_decay);
-
-// out[0] = wall-clock ticks slept (>= wall_ticks), out[1] = shader cycles over the same stretch
-hipError_t launch_clock_probe(hipStream_t stream, unsigned long long* out, unsigned long long wall_ticks);
 
 }  // namespace mcc

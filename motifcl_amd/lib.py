@@ -18,7 +18,6 @@ SIGNATURES = {
     "mcc_compact_counter_fused_workspace_nbytes": (_sz, [_sz, _sz, _sz]),
     "mcc_compact_counter_fused_strip_workspace_nbytes": (_sz, [_sz, _sz, _sz]),
     "mcc_compact_counter_fused_check": (ctypes.c_int, [_vp, _vp, _sz, _sz, _sz, _sz]),
-    "mcc_compact_counter_fused_strip_set_spin_limit": (None, [ctypes.c_uint]),
     "mcc_compact_counter_apply_update_fused": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
                        _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
@@ -46,14 +45,18 @@ SIGNATURES = {
     "mcc_memcpy_d2h": (ctypes.c_int, [_vp, _vp, _vp, _sz]),
     "mcc_memset_zero": (ctypes.c_int, [_vp, _vp, _sz]),
     "mcc_stream_synchronize": (ctypes.c_int, [_vp]),
-    "mcc_clock_probe": (ctypes.c_int, [_vp, _vp, _sz, ctypes.c_double]),
-    "mcc_wall_clock_khz": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int)]),
     "mcc_profiler_enable": (None, [ctypes.c_int]),
     "mcc_profiler_reset": (None, []),
     "mcc_profiler_query": (ctypes.c_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),
                                           ctypes.POINTER(ctypes.c_uint64)]),
 }
 
+# measurement and test aids: one entry per declaration in include/motifcl_amd_diag.h
+DIAG_SIGNATURES = {
+    "mcc_compact_counter_fused_strip_set_spin_limit": (None, [ctypes.c_uint]),
+    "mcc_clock_probe": (ctypes.c_int, [_vp, _vp, _sz, ctypes.c_double]),
+    "mcc_wall_clock_khz": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int)]),
+}
 
 
 class CounterTensor(ctypes.Structure):
@@ -90,7 +93,7 @@ def load():
             "%s is missing: build it with `python -m motifcl_amd.build` "
             "(or __graft_entry__.build())" % LIB_PATH)
     lib = ctypes.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in SIGNATURES.items():
+    for name, (restype, argtypes) in list(SIGNATURES.items()) + list(DIAG_SIGNATURES.items()):
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.restype = restype
         fn.argtypes = argtypes

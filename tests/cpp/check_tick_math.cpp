@@ -104,6 +104,26 @@ int main(int argc, char** argv) {
             return 2;
         }
     }
+    // first products by addition: (x ^ k) * M1 == x * M1 + hash_delta(x & 3, k)
+    for (long it = 0; it < 4000000; ++it) {
+        const uint32_t x = (uint32_t)next_u64();
+        for (uint32_t k = 0; k < 4; ++k)
+            if ((x ^ k) * mcc::kHashMul1 != x * mcc::kHashMul1 + mcc::hash_delta(x & 3u, k)) {
+                std::printf("hash_delta fails at %u^%u\n", x, k);
+                return 2;
+            }
+    }
+    // the per-row decision from the smallest magnitude agrees with the one from the key whenever it decides
+    for (long it = 0; it < 2000000; ++it) {
+        const float dn = log_uniform(1e-14, 1e14), ss = log_uniform(1e-30, 1e35);
+        float g = (next_u64() & 3) ? log_uniform(1e-45, 1e3) : 0.0f;
+        const int d = mcc::fast_division_from_min_abs(dn, ss, g);
+        const bool ref = mcc::row_takes_fast_division(dn, ss, mcc::range_key(g));
+        if ((d == 1 && !ref) || (d == -1 && ref && g != 0.0f) || (d == 0 && g != 0.0f)) {
+            std::printf("fast_division_from_min_abs disagrees dn=%a ss=%a g=%a\n", dn, ss, g);
+            return 2;
+        }
+    }
     // shared first hash step: (e + k) ^ ((e + k) >> 16) == (e ^ (e >> 16)) ^ k for e % 4 == 0
     for (long it = 0; it < 4000000; ++it) {
         const uint32_t e = (uint32_t)next_u64() & ~3u;

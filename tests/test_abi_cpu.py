@@ -22,11 +22,12 @@ def L():
 
 
 def test_every_declared_symbol_is_exported_and_bound(L):
-    header = open(os.path.join(ROOT, "include", "motifcl_amd.h")).read()
-    declared = set(re.findall(r"\b(mcc_[a-z0-9_]+)\s*\(", header))
-    assert declared == set(mlib.SIGNATURES), declared ^ set(mlib.SIGNATURES)
-    for name in declared:
-        assert hasattr(L, name)
+    for header_name, table in (("motifcl_amd.h", mlib.SIGNATURES), ("motifcl_amd_diag.h", mlib.DIAG_SIGNATURES)):
+        header = open(os.path.join(ROOT, "include", header_name)).read()
+        declared = set(re.findall(r"\b(mcc_[a-z0-9_]+)\s*\(", header))
+        assert declared == set(table), declared ^ set(table)
+        for name in declared:
+            assert hasattr(L, name)
 
 
 def _dense(L, C=11, n_in=8, n_out=2, lr=3e-3, lr_scale=0.0, beta=0.9, eps=1e-3,
