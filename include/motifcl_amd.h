@@ -154,6 +154,38 @@ int mcc_compact_counter_apply_update_fused(
     float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
 
 /*
+ * The fused step with the workspace inside the library: the same step as
+ * mcc_compact_counter_apply_update_fused, for callers that cannot allocate device
+ * memory -- code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  The workspace is a
+ * static device array of MCC_NOALLOC_WORKSPACE_NBYTES bytes that every GPU the
+ * library runs on holds from its first use there until the process ends; the
+ * call itself allocates nothing (no hipMalloc / hipFree, no stream-ordered
+ * allocation; with mcc_profiler_enable(1) the profiler may still create events).
+ * The step runs as mcc_compact_counter_apply_update_fused would with
+ *   - mcc_compact_counter_fused_workspace_nbytes(in, out, batch) bytes when that
+ *     fits the array (identical bytes to that call), else
+ *   - mcc_compact_counter_fused_strip_workspace_nbytes(in, out, batch) bytes when
+ *     the shape has a strip path and that fits (same restrictions: lr_scale == 0,
+ *     16-byte aligned x), else
+ *   - it fails with MCC_E_INVALID and a message that names both sizes.
+ * All calls on one GPU share that GPU's array, which keeps the last call's
+ * contents: two calls that overlap in time on one GPU (different streams) race.
+ * Arguments and validation are those of mcc_compact_counter_apply_update_fused
+ * without the workspace.
+ */
+#define MCC_NOALLOC_WORKSPACE_NBYTES ((size_t)32 << 20)
+int mcc_compact_counter_apply_update_fused_static(
+    void* stream,
+    uint8_t* state, size_t state_nbytes,
+    float* scale, size_t scale_nbytes,
+    float* v, size_t v_nbytes,
+    const float* grad_out, size_t grad_out_nbytes,
+    const float* x, size_t x_nbytes,
+    size_t C, size_t in_features, size_t out_features, size_t batch,
+    float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
+
+/*
  * The fused step for a list of tensors in a handful of launches: one grouped
  * contraction per tile size, one launch that adds the token-chunk slices, and
  * the batched update.  For models made of small layers (the 288- and 768-wide

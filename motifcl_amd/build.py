@@ -8,7 +8,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmotifcl_amd.so")
 
 SOURCES = ["capi.hip", "counter_update.hip", "gemm_tn_f32.hip", "gemm_tn_f32_wide.hip", "gemm_tn_bf16x6.hip", "counter_fused_strip.hip",
-           "counter_linear.hip", "counter_linear_bf16x3.hip", "side_optim.hip", "diag.hip"]
+           "counter_linear.hip", "counter_linear_bf16x3.hip", "side_optim.hip", "diag.hip", "noalloc.hip"]
 
 # -ffp-contract=off and correctly rounded divide/sqrt make every float operation a single
 # IEEE-754 binary32 rounding, which the bit-exact update relies on.  Packed fp32 ops are

@@ -269,14 +269,14 @@ int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t 
     return MCC_OK;
 }
 
-int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t state_nbytes,
-                                           float* scale, size_t scale_nbytes, float* v,
-                                           size_t v_nbytes, const float* grad_out,
-                                           size_t grad_out_nbytes, const float* x, size_t x_nbytes,
-                                           void* workspace, size_t workspace_nbytes, size_t C,
-                                           size_t in_features, size_t out_features, size_t batch,
-                                           float lr, float lr_scale, float rms_beta, float rms_eps,
-                                           uint32_t seed) {
+}  // extern "C"
+
+// Validation and launches of the fused step, shared by mcc_compact_counter_apply_update_fused and
+// the entry point that brings its own workspace (noalloc.hip).  Allocates nothing on the device.
+int mcc::fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* scale, size_t scale_nbytes, float* v,
+                      size_t v_nbytes, const float* grad_out, size_t grad_out_nbytes, const float* x, size_t x_nbytes,
+                      void* workspace, size_t workspace_nbytes, size_t C, size_t in_features, size_t out_features,
+                      size_t batch, float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed) {
     const char* what = "compact-counter fused update";
     if (batch == 0) return fail(MCC_E_INVALID, "compact-counter fused update requires non-zero dimensions");
     if (!check_codec(what, C, in_features, out_features)) return MCC_E_INVALID;
@@ -338,6 +338,21 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
     }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update launch failed");
     return MCC_OK;
+}
+
+extern "C" {
+
+int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t state_nbytes,
+                                           float* scale, size_t scale_nbytes, float* v,
+                                           size_t v_nbytes, const float* grad_out,
+                                           size_t grad_out_nbytes, const float* x, size_t x_nbytes,
+                                           void* workspace, size_t workspace_nbytes, size_t C,
+                                           size_t in_features, size_t out_features, size_t batch,
+                                           float lr, float lr_scale, float rms_beta, float rms_eps,
+                                           uint32_t seed) {
+    return mcc::fused_update(stream, state, state_nbytes, scale, scale_nbytes, v, v_nbytes, grad_out, grad_out_nbytes, x,
+                             x_nbytes, workspace, workspace_nbytes, C, in_features, out_features, batch, lr, lr_scale,
+                             rms_beta, rms_eps, seed);
 }
 
 // Where tensor i's slices start in a batched fused workspace: each tensor gets what

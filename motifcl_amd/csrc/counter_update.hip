@@ -769,9 +769,24 @@ hipError_t launch_update_batch(hipStream_t stream, const UpdateTensor* tensors, 
     a.cd = make_codec(C);
     a.geom = lut_geom(a.cd);
     a.lr_scale = lr_scale; a.rms_beta = rms_beta; a.rms_eps = rms_eps;
-    std::vector<int> cls(n);
-    std::vector<char> done(n, 0);
-    for (size_t i = 0; i < n; ++i) cls[i] = iters_class(tensors[i]);
+    // short lists (one tensor, a layer, a small model) are sorted on the stack: no host allocation
+    constexpr size_t kOnStack = 256;
+    int cls_stack[kOnStack];
+    char done_stack[kOnStack];
+    std::vector<int> cls_heap;
+    std::vector<char> done_heap;
+    int* cls = cls_stack;
+    char* done = done_stack;
+    if (n > kOnStack) {
+        cls_heap.resize(n);
+        done_heap.resize(n);
+        cls = cls_heap.data();
+        done = done_heap.data();
+    }
+    for (size_t i = 0; i < n; ++i) {
+        cls[i] = iters_class(tensors[i]);
+        done[i] = 0;
+    }
     for (size_t i = 0; i < n; ++i) {
         if (done[i]) continue;
         a.n_tensors = 0;

@@ -13,6 +13,13 @@ namespace mcc {
 int report_failure(int code, const std::string& message);
 int report_hip_failure(hipError_t e, const char* what);
 
+// The fused step behind mcc_compact_counter_apply_update_fused (capi.hip): validates, then
+// enqueues; `workspace_nbytes` selects the two-kernel or the strip path.
+int fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* scale, size_t scale_nbytes, float* v,
+                 size_t v_nbytes, const float* grad_out, size_t grad_out_nbytes, const float* x, size_t x_nbytes,
+                 void* workspace, size_t workspace_nbytes, size_t C, size_t in_features, size_t out_features,
+                 size_t batch, float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed);
+
 // One counter tensor of an update-only batch (device pointers).
 struct UpdateTensor {
     uint8_t* state;

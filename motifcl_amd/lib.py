@@ -21,6 +21,9 @@ SIGNATURES = {
     "mcc_compact_counter_apply_update_fused": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
                        _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
+    "mcc_compact_counter_apply_update_fused_static": (
+        ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz,
+                       _sz, _sz, _sz, _sz, _f, _f, _f, _f, _u32]),
     "mcc_compact_counter_fused_batched_workspace_nbytes": (_sz, [_vp, _sz]),
     "mcc_compact_counter_apply_update_fused_batched": (
         ctypes.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _f, _f, _f]),

@@ -134,6 +134,22 @@ def apply_update_fused(state, scale, v, grad_out, x, workspace, C, lr, lr_scale,
         C, in_features, out_features, batch, lr, lr_scale, rms_beta, rms_eps, seed & 0xFFFFFFFF))
 
 
+NOALLOC_WORKSPACE_NBYTES = 32 << 20  # MCC_NOALLOC_WORKSPACE_NBYTES of include/motifcl_amd.h
+
+
+def apply_update_fused_static(state, scale, v, grad_out, x, C, lr, lr_scale, rms_beta, rms_eps, seed):
+    """The fused step on the library's own static workspace: the call allocates nothing."""
+    L = _lib.load()
+    batch, out_features = grad_out.shape
+    in_features = x.shape[1]
+    if x.shape[0] != batch:
+        raise ValueError("x and grad_out disagree on the batch size")
+    _lib.check(L.mcc_compact_counter_apply_update_fused_static(
+        _stream(), *_buf(state, torch.uint8), *_buf(scale, torch.float32), *_buf(v, torch.float32),
+        *_buf(grad_out, torch.float32), *_buf(x, torch.float32),
+        C, in_features, out_features, batch, lr, lr_scale, rms_beta, rms_eps, seed & 0xFFFFFFFF))
+
+
 def matmul_transpose_a(a, b, out=None):
     """c[m,n] = a[k,m]^T . b[k,n]."""
     L = _lib.load()
