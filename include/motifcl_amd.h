@@ -93,19 +93,30 @@ size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out
                                                   size_t batch);
 
 /*
- * Bytes of the small workspace of the accumulator-resident fused step
- * (32 KiB per 128 output rows plus flags), or 0 when the shape is not
- * supported by it.  No counterpart in the reference.
+ * Bytes of the small workspace with which mcc_compact_counter_apply_update_fused
+ * runs without a buffer of the size of the weight gradient, or 0 when the shape
+ * has no way smaller than the full workspace (tiny layers).  Layers whose in and
+ * out are multiples of 128 with in >= 768 take the accumulator-resident strip
+ * path: 512 bytes of partial row sums per output row plus a few control words
+ * (5.6 MB for the largest layer of a 7B model instead of 180 MB).  Every other shape
+ * is updated band by band of an eighth of its output rows: the workspace holds
+ * one band's gradient.  No counterpart in the reference, whose fused kernels
+ * recompute the gradient instead of holding it.
  */
 size_t mcc_compact_counter_fused_strip_workspace_nbytes(size_t in_features, size_t out_features,
                                                         size_t batch);
 
 /*
- * Waits for `stream` and reports whether the last fused step that used
- * `workspace` completed: MCC_OK, or MCC_E_RUNTIME when a strip-workspace
- * step gave up a wait (state of that tensor is then partially updated).
- * Always MCC_OK for the full-size workspace.  No counterpart in the
- * reference.
+ * Waits for `stream` and reports whether every strip-path step of this process
+ * on the current GPU since the last call completed: MCC_OK, or MCC_E_RUNTIME
+ * when a step gave up a wait between tiles.  Such a step leaves whole 128-row
+ * strips of its tensor without their update -- state, scale and v of those rows
+ * are untouched, no strip is half-updated -- and the report clears the count.
+ * The count lives in the library, per GPU, so it survives other layers' steps
+ * through the same workspace; the workspace and shape arguments are not looked
+ * at (kept for callers written against the first form of this call).  Always
+ * MCC_OK for steps on the full workspace or band by band.  No counterpart in
+ * the reference.
  */
 int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t workspace_nbytes,
                                     size_t in_features, size_t out_features, size_t batch);
@@ -122,21 +133,23 @@ int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t 
  *   - >= mcc_compact_counter_fused_workspace_nbytes (one f32[out,in] slice
  *     per token chunk of the contraction; large layers have one chunk):
  *     contraction into the workspace, then the update kernel.  After the call
- *     the first out*in floats of the workspace hold grad_w.
+ *     the first out*in floats of the workspace hold grad_w.  The fastest way.
  *   - >= mcc_compact_counter_fused_strip_workspace_nbytes but smaller than
- *     the above: the update is applied from the contraction's accumulators
- *     and no weight-sized buffer exists at any time, which is the property
- *     tests/test_memory_truth_gate.cpp:109-113 of the reference asks for.
- *     Needs lr_scale == 0, in/out multiples of 128 and a 16-byte aligned x.
- *     Tiles of one row strip wait for each other on the device; two such
- *     calls must not run concurrently on one GPU (they could starve each
- *     other's waits), and mcc_compact_counter_fused_check reports a wait
- *     that was given up.
- * Both ways produce identical bytes whenever the first does not split the
- * tokens into chunks, i.e. for fewer than 512 tokens or layers of at least
- * 1024 tiles of 128 x 128 (mcc_compact_counter_fused_workspace_nbytes ==
- * out*in*4); where it does, its gradient is the sum of chunk sums and the two
- * ways differ by that rounding (a few counters in 10^5 flip differently).
+ *     the above: no weight-sized buffer exists at any time, which is the
+ *     property tests/test_memory_truth_gate.cpp:109-113 of the reference asks
+ *     for.  Any lr_scale.  On the strip path (see the size query) the update is
+ *     applied from the contraction's accumulators; x must be 16-byte aligned;
+ *     tiles of one row strip wait for each other on the device, so a second
+ *     such call issued on another stream while one is still running is refused
+ *     with MCC_E_INVALID (order the two), every wait is bounded, and
+ *     mcc_compact_counter_fused_check reports a wait that was given up.  On a
+ *     stream under graph capture the refusal is not applied: do not replay two
+ *     such graphs side by side.
+ * The ways produce identical bytes whenever none of them splits the tokens into
+ * chunks, i.e. for fewer than 512 tokens or layers of at least 1024 tiles of
+ * 128 x 128 (mcc_compact_counter_fused_workspace_nbytes == out*in*4); where
+ * one does, its gradient is the sum of chunk sums and they differ by that
+ * rounding (a few counters in 10^5 flip differently).
  * grad_w differs from the reference's
  * sequential fp32 sum only by summation order (relative error <= 1e-4 of the
  * row norm); given that grad_w the counter arithmetic is the same as in the
@@ -166,8 +179,7 @@ int mcc_compact_counter_apply_update_fused(
  *   - mcc_compact_counter_fused_workspace_nbytes(in, out, batch) bytes when that
  *     fits the array (identical bytes to that call), else
  *   - mcc_compact_counter_fused_strip_workspace_nbytes(in, out, batch) bytes when
- *     the shape has a strip path and that fits (same restrictions: lr_scale == 0,
- *     16-byte aligned x), else
+ *     that fits, else
  *   - it fails with MCC_E_INVALID and a message that names both sizes.
  * All calls on one GPU share that GPU's array, which keeps the last call's
  * contents: two calls that overlap in time on one GPU (different streams) race.

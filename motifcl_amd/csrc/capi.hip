@@ -4,6 +4,7 @@
 // failures are reported, never thrown, and enqueue nothing.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdint>
@@ -68,6 +69,13 @@ bool check_codec(const char* what, size_t C, size_t in_features, size_t out_feat
         return false;
     }
     return true;
+}
+
+// True when two entries of `states` are the same pointer: descriptors that share a state would be
+// updated by several workgroups of one launch at once.
+bool has_duplicate(std::vector<const void*> states) {
+    std::sort(states.begin(), states.end());
+    return std::adjacent_find(states.begin(), states.end()) != states.end();
 }
 
 // ---- pooled device storage -------------------------------------------------
@@ -198,7 +206,7 @@ static int check_update_tensor(const mcc_counter_tensor& t, size_t C, float lr_s
         return fail(MCC_E_INVALID, "compact-counter update float buffers must be 4-byte aligned");
     out->state = t.state; out->scale = t.scale; out->v = t.v; out->grad_w = t.grad_w;
     out->in_features = (int)t.in_features; out->out_features = (int)t.out_features;
-    out->row_start = 0; out->seed = t.seed; out->lr = t.lr; out->pad = 0;
+    out->row_start = 0; out->seed = t.seed; out->lr = t.lr; out->first_row = 0;
     return MCC_OK;
 }
 
@@ -226,6 +234,12 @@ int mcc_compact_counter_apply_update_dense_batched(void* stream, const mcc_count
             return rc;
         }
     }
+    if (n_tensors > 1) {
+        std::vector<const void*> states(n_tensors);
+        for (size_t i = 0; i < n_tensors; ++i) states[i] = tensors[i].state;
+        if (has_duplicate(std::move(states)))
+            return fail(MCC_E_INVALID, "compact-counter update received the same state twice in one list");
+    }
     hipError_t e;
     {
         ScopedKernelTimer timer("counter_update", static_cast<hipStream_t>(stream));
@@ -246,26 +260,76 @@ size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out
     return slices * out_features * in_features * sizeof(float);
 }
 
+}  // extern "C"
+
+namespace {
+
+// How the fused step runs on a workspace smaller than the full one:
+//   strip   the accumulator-resident kernel (in/out multiples of 128, rows of at least 768 weights:
+//           its 512 bytes of partial sums per output row are then at most a sixth of the row);
+//   banded  the two-kernel path applied to bands of `band_rows` output rows, one after the other
+//           through a workspace of an eighth of the weight gradient -- any shape, slower (the bands
+//           are small contractions), for the layers too small or too oddly shaped for the strips.
+struct SmallPlan {
+    enum Kind { kNone, kStrip, kBanded } kind = kNone;
+    size_t nbytes = 0;
+    int band_rows = 0;
+    mcc::GemmTnPlan band_plan{};
+};
+
+SmallPlan small_workspace_plan(size_t in_features, size_t out_features, size_t batch) {
+    SmallPlan p;
+    if (in_features == 0 || out_features == 0 || batch == 0 || in_features % 4 != 0) return p;
+    if (in_features > kIntMax || out_features > kIntMax || batch > kIntMax) return p;
+    if (in_features >= 768 && mcc::fused_strip_supports(in_features, out_features, batch)) {
+        p.kind = SmallPlan::kStrip;
+        p.nbytes = mcc::fused_strip_workspace_nbytes(in_features, out_features, batch);
+        return p;
+    }
+    // rows x token chunks the workspace may hold: an eighth of the gradient, so that a caller whose
+    // allocator rounds up to a power of two still stays below a quarter
+    const size_t budget_rows = out_features / 8 > 0 ? out_features / 8 : 1;
+    size_t rows = budget_rows >= 8 ? budget_rows / 8 * 8 : budget_rows;
+    mcc::GemmTnPlan plan = mcc::plan_gemm_tn((int)batch, (int)rows, (int)in_features);
+    if ((size_t)plan.splits * rows > budget_rows) {
+        // fewer token chunks than the band would take on its own
+        const size_t splits = budget_rows / rows > 0 ? budget_rows / rows : 1;
+        int chunk = (int)((batch + splits - 1) / splits);
+        chunk = (chunk + 15) / 16 * 16;
+        plan.chunk = chunk;
+        plan.splits = (int)((batch + chunk - 1) / chunk);
+    }
+    p.kind = SmallPlan::kBanded;
+    p.band_rows = (int)rows;
+    p.band_plan = plan;
+    p.nbytes = ((size_t)plan.splits * rows * in_features * sizeof(float) + 255) / 256 * 256;
+    return p;
+}
+
+}  // namespace
+
+extern "C" {
+
 size_t mcc_compact_counter_fused_strip_workspace_nbytes(size_t in_features, size_t out_features,
                                                         size_t batch) {
-    return mcc::fused_strip_workspace_nbytes(in_features, out_features, batch);
+    const SmallPlan p = small_workspace_plan(in_features, out_features, batch);
+    const size_t full = mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch);
+    return p.kind != SmallPlan::kNone && p.nbytes < full ? p.nbytes : 0;
 }
 
 int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t workspace_nbytes,
                                     size_t in_features, size_t out_features, size_t batch) {
-    if (!workspace) return fail(MCC_E_INVALID, "compact-counter fused check received a null workspace");
+    (void)workspace; (void)workspace_nbytes; (void)in_features; (void)out_features; (void)batch;
     const hipError_t es = hipStreamSynchronize(static_cast<hipStream_t>(stream));
     if (es != hipSuccess) return hip_fail(es, "compact-counter fused check: stream synchronize failed");
-    const size_t full_nbytes = mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch);
-    if (full_nbytes == 0) return fail(MCC_E_INVALID, "compact-counter fused check requires non-zero dimensions");
-    if (workspace_nbytes >= full_nbytes) return MCC_OK;  // two-kernel path: nothing to wait on across workgroups
-    int status = 0;
-    const hipError_t ec = hipMemcpy(&status, workspace, sizeof(int), hipMemcpyDeviceToHost);
+    int failures = 0;
+    const hipError_t ec = mcc::fused_strip_take_failures(&failures);
     if (ec != hipSuccess) return hip_fail(ec, "compact-counter fused check: status read failed");
-    if (status != 0)
+    if (failures != 0)
         return fail(MCC_E_RUNTIME,
-                    "compact-counter fused strip update gave up waiting for a neighbouring tile; "
-                    "state, scale and v of this tensor are partially updated");
+                    "compact-counter fused strip update gave up waiting for a neighbouring tile in " +
+                        std::to_string(failures) + " launch(es) on this GPU since the last check; in such a launch "
+                        "whole 128-row strips of the tensor are left without their update (no strip is half-updated)");
     return MCC_OK;
 }
 
@@ -298,14 +362,13 @@ int mcc::fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* 
     if (grad_out_nbytes < batch * out_features * sizeof(float) || x_nbytes < batch * in_features * sizeof(float))
         return fail(MCC_E_INVALID, "compact-counter fused update activation buffer is too small");
     const size_t full_nbytes = mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch);
-    const size_t strip_nbytes = mcc::fused_strip_workspace_nbytes(in_features, out_features, batch);
-    const bool strip_path = workspace_nbytes < full_nbytes;
-    if (strip_path) {
-        if (strip_nbytes == 0 || workspace_nbytes < strip_nbytes)
+    const bool small = workspace_nbytes < full_nbytes;
+    SmallPlan plan;
+    if (small) {
+        plan = small_workspace_plan(in_features, out_features, batch);
+        if (plan.kind == SmallPlan::kNone || workspace_nbytes < plan.nbytes)
             return fail(MCC_E_INVALID, "compact-counter fused update workspace is too small");
-        if (lr_scale != 0.0f)
-            return fail(MCC_E_INVALID, "compact-counter fused update with the strip workspace requires lr_scale == 0");
-        if (reinterpret_cast<uintptr_t>(x) % 16)
+        if (plan.kind == SmallPlan::kStrip && reinterpret_cast<uintptr_t>(x) % 16)
             return fail(MCC_E_INVALID, "compact-counter fused update with the strip workspace requires 16-byte aligned x");
     }
     if (reinterpret_cast<uintptr_t>(workspace) % 16)
@@ -316,12 +379,37 @@ int mcc::fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* 
     hipStream_t s = static_cast<hipStream_t>(stream);
     float* grad_w = static_cast<float*>(workspace);
     hipError_t e;
-    if (strip_path) {
+    if (small && plan.kind == SmallPlan::kStrip) {
         ScopedKernelTimer timer("fused_strip", s);
+        bool busy = false;
         e = mcc::launch_fused_strip(s, state, scale, v, grad_out, x, workspace, (int)C, (int)in_features,
-                                    (int)out_features, (int)batch, lr, rms_beta, rms_eps, seed,
-                                    mcc::fused_strip_spin_limit());
+                                    (int)out_features, (int)batch, lr, lr_scale, rms_beta, rms_eps, seed,
+                                    mcc::fused_strip_spin_limit(), &busy);
         if (e != hipSuccess) return hip_fail(e, "compact-counter fused strip update launch failed");
+        if (busy)
+            return fail(MCC_E_INVALID,
+                        "compact-counter fused update with the strip workspace: another such step is still running on a "
+                        "different stream of this GPU; order the two (one stream, or an event between them)");
+        return MCC_OK;
+    }
+    if (small) {
+        // band after band: contraction of the band's rows into the workspace, then their update
+        const size_t groups_per_row = in_features / 4;
+        for (size_t r0 = 0; r0 < out_features; r0 += (size_t)plan.band_rows) {
+            const size_t rows = out_features - r0 < (size_t)plan.band_rows ? out_features - r0 : (size_t)plan.band_rows;
+            {
+                ScopedKernelTimer timer("gemm_tn_f32", s);
+                e = mcc::launch_gemm_tn_f32(s, grad_out + r0, x, grad_w, (int)batch, (int)rows, (int)in_features, grad_w, 0,
+                                            (int)out_features, &plan.band_plan);
+            }
+            if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
+            {
+                ScopedKernelTimer timer("counter_update", s);
+                e = mcc::launch_update_dense(s, state + r0 * groups_per_row * 3, scale + r0, v + r0, grad_w, (int)C,
+                                             (int)in_features, (int)rows, lr, lr_scale, rms_beta, rms_eps, seed, (int)r0);
+            }
+            if (e != hipSuccess) return hip_fail(e, "compact-counter fused update launch failed");
+        }
         return MCC_OK;
     }
     {
@@ -385,24 +473,6 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
     if (need == 0) return fail(MCC_E_INVALID, "compact-counter fused update requires non-zero dimensions");
     if (workspace_nbytes < need) return fail(MCC_E_INVALID, "compact-counter fused update workspace is too small");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // another contraction mode than the fp32 instruction: tensor by tensor, each in its own region
-    if (g_contraction_mode.load() != MCC_CONTRACTION_FP32) {
-        uint8_t* ws = static_cast<uint8_t*>(workspace);
-        for (size_t i = 0; i < n_tensors; ++i) {
-            const mcc_fused_tensor& t = tensors[i];
-            const size_t region = fused_batched_region(t);
-            const int rc = mcc_compact_counter_apply_update_fused(
-                stream, t.state, t.state_nbytes, t.scale, t.scale_nbytes, t.v, t.v_nbytes, t.grad_out, t.grad_out_nbytes,
-                t.x, t.x_nbytes, ws, region, C, t.in_features, t.out_features, t.batch, t.lr, lr_scale, rms_beta,
-                rms_eps, t.seed);
-            if (rc != MCC_OK) {
-                g_error = "tensor " + std::to_string(i) + ": " + g_error;
-                return rc;
-            }
-            ws += region;
-        }
-        return MCC_OK;
-    }
     std::vector<mcc::GemmTnJob> jobs(n_tensors);
     std::vector<mcc::UpdateTensor> upd(n_tensors);
     uint8_t* ws = static_cast<uint8_t*>(workspace);
@@ -443,6 +513,31 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
         jobs[i].m = (int)t.out_features;
         jobs[i].n = (int)t.in_features;
         ws += fused_batched_region(t);
+    }
+    if (n_tensors > 1) {
+        std::vector<const void*> states(n_tensors);
+        for (size_t i = 0; i < n_tensors; ++i) states[i] = tensors[i].state;
+        if (has_duplicate(std::move(states)))
+            return fail(MCC_E_INVALID, "compact-counter fused update received the same state twice in one list");
+    }
+    // every tensor has been validated: nothing below fails for a reason the arguments could show
+    // another contraction mode than the fp32 instruction: tensor by tensor, each in its own region
+    if (g_contraction_mode.load() != MCC_CONTRACTION_FP32) {
+        ws = static_cast<uint8_t*>(workspace);
+        for (size_t i = 0; i < n_tensors; ++i) {
+            const mcc_fused_tensor& t = tensors[i];
+            const size_t region = fused_batched_region(t);
+            const int rc = mcc_compact_counter_apply_update_fused(
+                stream, t.state, t.state_nbytes, t.scale, t.scale_nbytes, t.v, t.v_nbytes, t.grad_out, t.grad_out_nbytes,
+                t.x, t.x_nbytes, ws, region, C, t.in_features, t.out_features, t.batch, t.lr, lr_scale, rms_beta,
+                rms_eps, t.seed);
+            if (rc != MCC_OK) {
+                g_error = "tensor " + std::to_string(i) + ": " + g_error;
+                return rc;
+            }
+            ws += region;
+        }
+        return MCC_OK;
     }
     hipError_t e;
     {

@@ -31,6 +31,7 @@
 
 #include <atomic>
 #include <cstdint>
+#include <mutex>
 
 #include "counter_math.hpp"
 #include "gemm_tile.hpp"
@@ -43,7 +44,17 @@ namespace {
 constexpr int kTile = 128;             // rows and columns of G per tile
 constexpr int kGroupsPerTile = kTile / 4;
 constexpr int kNapsPerHandOff = 2;  // s_sleep(32) units (about 0.9 us each) slept per pending hand-off
-constexpr int kStripChainFloats = 2 * kTile * kGroupsPerTile;  // both parities, 128 rows x 32 chains
+constexpr int kChainSetFloats = 2 * kTile * kGroupsPerTile;  // both parities, 128 rows x 32 chains
+constexpr int kStripChainFloats = 2 * kChainSetFloats;       // the sums of g^2 and of g*t
+
+// Per-strip control words.  A strip is updated all or nothing: `decision` goes from 0 to +1 when
+// both hand-off sequences have reached the end of the strip (set by the tile that completes the
+// second one) or to -1 when a tile gives up; no tile writes a tick, v or scale before it has read +1.
+struct StripControl {
+    int published[2];  // tiles of each parity that have published their chains
+    int sequences_done;
+    int decision;
+};
 
 struct StripArgs {
     uint8_t* state;
@@ -51,16 +62,17 @@ struct StripArgs {
     float* v;
     const float* grad_out;
     const float* x;
-    int* status;   // 0 while healthy
-    int* flags;    // [strip][2]: tiles of each parity that have published their chains
-    float* chain;  // [strip][2][128][32]
+    int* status;            // launch-local: raised by the first workgroup that gives up, ends all waits
+    int* failures;          // the library's per-device count of strip launches' workgroups that gave up
+    StripControl* control;  // [strip]
+    float* chain;           // [strip][g^2, g*t][parity][128][32]
     int tokens, in_features, out_features;
     int tiles_per_strip, total_tiles;
     int layer_wgs;  // workgroups the device takes in per residency layer (its CU count)
     unsigned spin_limit;
     Codec cd;
     LutGeom geom;
-    float lr, rms_beta, rms_eps;
+    float lr, lr_scale, rms_beta, rms_eps;
     uint32_t seed;
 };
 
@@ -153,28 +165,44 @@ __device__ __forceinline__ TilePos fresh_tile_pos() {
     return p;
 }
 
-// Thread 0 polls until *flag >= want or the status word is raised; returns whether the
-// workgroup may go on.  All threads of the workgroup call it.
-__device__ __forceinline__ bool wait_for(const StripArgs& a, const int* flag, int want, EpilogueLds& e) {
+__device__ __forceinline__ bool cas_relaxed(int* p, int expected, int desired) {
+    return __hip_atomic_compare_exchange_strong(p, &expected, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// A workgroup that cannot go on: the strip is marked aborted unless it has been committed already,
+// the launch-local status ends every other wait, and the library's failure count remembers it.
+// Returns the strip's final decision (+1 if the commit came first).
+__device__ __forceinline__ int give_up(const StripArgs& a, StripControl* c) {
+    cas_relaxed(&c->decision, 0, -1);
+    const int d = load_relaxed(&c->decision);
+    if (d < 0) {
+        if (__hip_atomic_exchange(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+            __hip_atomic_fetch_add(a.failures, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return d;
+}
+
+// Thread 0 polls until *word >= want (a hand-off counter) or, with DECISION, until *word != 0,
+// the status word is raised, or the spin budget is spent; e.ok tells the workgroup whether the
+// condition came true.  All threads of the workgroup call it.
+template <bool DECISION>
+__device__ __forceinline__ bool wait_for(const StripArgs& a, const int* word, int want, EpilogueLds& e) {
     if (threadIdx.x == 0) {
         int ok = 1;
         unsigned spins = 0, polls = 0;
-        int seen;
-        while ((seen = load_relaxed(flag)) < want) {
-            // The flag counts hand-offs, each of which takes a few microseconds: sleep in
+        for (;;) {
+            const int seen = load_relaxed(word);
+            if (DECISION ? seen != 0 : seen >= want) break;
+            // A hand-off counter counts hand-offs, each of which takes a few microseconds: sleep in
             // proportion to the hand-offs still to come instead of polling at full rate.  A
             // thousand workgroups polling a handful of words slow the contractions that are
             // still running by a third.
-            const int naps = (want - seen - 1) * kNapsPerHandOff;
+            const int naps = DECISION ? 0 : (want - seen - 1) * kNapsPerHandOff;
             __builtin_amdgcn_s_sleep(8);
             for (int n = 0; n < naps; ++n) __builtin_amdgcn_s_sleep(32);
             spins += 1u + (unsigned)naps;
-            if ((++polls & 15u) == 0 && load_relaxed(a.status) != 0) {
-                ok = 0;
-                break;
-            }
-            if (spins >= a.spin_limit) {
-                __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (((++polls & 15u) == 0 && load_relaxed(a.status) != 0) || spins >= a.spin_limit) {
                 ok = 0;
                 break;
             }
@@ -187,8 +215,35 @@ __device__ __forceinline__ bool wait_for(const StripArgs& a, const int* flag, in
     return ok;
 }
 
+// One chain step of the hand-off for one of the two sums: every lane adds the four values of its
+// packed group to the chain slot of (row, group) in element order.  `value(i, j, r)` is this
+// lane's value for accumulator element (i, j, r).
+template <typename Value>
+__device__ __forceinline__ void chain_step(float* lds, const TilePos& tp, int kq, Value value) {
+    using Cfg = TileCfg<kTile, kTile>;
+#pragma unroll
+    for (int i = 0; i < Cfg::kTilesM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = tp.wm0 + 32 * i + 8 * (r / 4) + 4 * tp.half + (r % 4);
+#pragma unroll
+            for (int j = 0; j < Cfg::kTilesN; ++j) {
+                const int gi = (tp.wn0 + 32 * j + tp.l32) >> 2;
+                float* slot = lds + row * kGroupsPerTile + gi;  // owned by this lane's quad
+                float c = *slot;
+                const float val = value(i, j, r);
+                c = c + quad_lane<0>(val);  // element order inside the group
+                c = c + quad_lane<1>(val);
+                c = c + quad_lane<2>(val);
+                c = c + quad_lane<3>(val);
+                if (kq == 0) *slot = c;
+            }
+        }
+}
+
 // DIRECT: tokens % 16 == 0 and grad_out 16-byte aligned, so the slabs can go straight to LDS.
-template <bool VEC_A, bool DIRECT>
+// WITH_GS: lr_scale != 0, the row sums of g * t travel beside the sums of squares.
+template <bool VEC_A, bool DIRECT, bool WITH_GS>
 __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs a) {
     using Cfg = TileCfg<kTile, kTile>;
     __shared__ float lds[DIRECT ? DirectCfg<kTile, kTile>::kLdsFloats : Cfg::kLdsFloats];
@@ -203,24 +258,33 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
 
     const int groups_per_row = a.in_features >> 2;
     const uint32_t last_group_off = 3u * ((uint32_t)a.out_features * (uint32_t)groups_per_row - 1u);
+    const uint32_t row_bytes = 3u * (uint32_t)groups_per_row;
 
     for (int tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
+        // once a workgroup has given up nothing new is started: a strip whose tiles have not all
+        // published cannot have been committed, and this tile has not published yet
+        if (threadIdx.x == 0) e.ok = load_relaxed(a.status) == 0 ? 1 : 0;
+        __syncthreads();
+        const bool healthy = e.ok != 0;
+        __syncthreads();
+        if (!healthy) return;
         const int strip = tile / a.tiles_per_strip;
         const int ct = tile - strip * a.tiles_per_strip;
         const int m0 = strip * kTile, n0 = ct * kTile;
         const int parity = ct & 1, step = ct >> 1;
-        int* flags = a.flags + 2 * strip;
+        StripControl* control = a.control + strip;
         float* chain = a.chain + (size_t)strip * kStripChainFloats;
 
         floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
         // even progress of the workgroups that share a CU: a strip is as slow as its slowest tile
         if (DIRECT)
             gemm_tile_mainloop_direct<kTile, kTile, true>(a.grad_out, a.x, a.tokens, a.out_features, a.in_features,
-                                                          m0, n0, tp0, lds, acc, (int)blockIdx.x / a.layer_wgs);
+                                                          m0, n0, tp0, lds, acc, a.out_features,
+                                                          (int)blockIdx.x / a.layer_wgs);
         else
             gemm_tile_mainloop<kTile, kTile, VEC_A, true, true>(a.grad_out, a.x, a.tokens, a.out_features,
                                                                 a.in_features, m0, n0, tp0, lds, acc,
-                                                                (int)blockIdx.x / a.layer_wgs);
+                                                                a.out_features, (int)blockIdx.x / a.layer_wgs);
 
         park_accumulators(acc);
         // the hand-off sequence is latency-bound and other workgroups of this CU are still in
@@ -230,83 +294,116 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         int lane = tp.tid & 63, wave = tp.tid >> 6;
         int kq = tp.l32 & 3;  // position of this lane's column inside its packed group
 
-        // Old per-row values, read before this tile publishes anything: tile 0 overwrites them
-        // only after every tile of the strip has published.
+        // Old per-row values, read before anything of this strip is written: tile 0 overwrites
+        // them only after the strip has been committed, and commits happen after every tile of
+        // the strip has been here.
         float s_old = 0.0f, v_old = 0.0f;
         if (tp.tid < kTile) {
             s_old = a.scale[m0 + tp.tid];
             v_old = a.v[m0 + tp.tid];
         }
+        // byte offsets of this thread's accumulator elements from the state base (the launch checks
+        // that the state is smaller than 2 GiB) and their element indices
+        const uint32_t my_state = (uint32_t)(m0 + tp.wm0 + 4 * tp.half) * row_bytes +
+                                  3u * ((uint32_t)(n0 + tp.wn0 + tp.l32) >> 2);
+        // One 4-byte load per lane and element; the tensor's last group has no byte after it, so it
+        // is fetched one byte early and shifted down.
+        auto load_word = [&](int i, int j, int r) {
+            const uint32_t off = my_state + (uint32_t)(32 * i + 8 * (r / 4) + (r % 4)) * row_bytes + 24u * j;
+            const uint32_t is_last = off == last_group_off ? 1u : 0u;
+            uint32_t word;
+            __builtin_memcpy(&word, a.state + (off - is_last), 4);
+            return word >> (8 * is_last);
+        };
 
         // ---- chain hand-off: step `step` of chains 32*parity .. 32*parity+31 -------------
-        // The 128 x 32 chain block (16 KiB) is staged in the contraction's LDS slab buffer, which
-        // is free by now; each thread moves 16 floats, 256 contiguous bytes per wave and access.
-        if (!wait_for(a, flags + parity, step, e)) return;
+        // The 128 x 32 chain block (16 KiB per sum) is staged in the contraction's LDS slab buffer,
+        // which is free by now; each thread moves 16 floats, 256 contiguous bytes per wave and access.
+        if (!wait_for<false>(a, &control->published[parity], step, e)) {
+            if (threadIdx.x == 0) give_up(a, control);
+            return;
+        }
         park_accumulators(acc);
-        float* my_chain = chain + parity * (kTile * kGroupsPerTile);
         static_assert(Cfg::kLdsFloats >= kTile * kGroupsPerTile, "chain block must fit the slab buffer");
         constexpr int kChainPerThread = kTile * kGroupsPerTile / kGemmThreads;
-        {
-            float in[kChainPerThread];
+#pragma unroll
+        for (int set = 0; set < (WITH_GS ? 2 : 1); ++set) {
+            float* my_chain = chain + set * kChainSetFloats + parity * (kTile * kGroupsPerTile);
+            {
+                float in[kChainPerThread];
+#pragma unroll
+                for (int p = 0; p < kChainPerThread; ++p)
+                    in[p] = step > 0 ? load_shared_f32(my_chain + tp.tid + kGemmThreads * p) : 0.0f;
+#pragma unroll
+                for (int p = 0; p < kChainPerThread; ++p) lds[tp.tid + kGemmThreads * p] = in[p];
+            }
+            __syncthreads();
+            if (set == 0) {
+                chain_step(lds, tp, kq, [&](int i, int j, int r) { return acc[i][j][r] * acc[i][j][r]; });
+            } else {
+                // g * t (kernels/compact_counter.cl:81-82): t from this element's code
+                chain_step(lds, tp, kq, [&](int i, int j, int r) {
+                    const uint32_t code = (load_word(i, j, r) >> (6 * kq)) & 0x3fu;
+                    return acc[i][j][r] * (float)(code_q(code, a.cd) - 1);
+                });
+            }
+            __syncthreads();
 #pragma unroll
             for (int p = 0; p < kChainPerThread; ++p)
-                in[p] = step > 0 ? load_shared_f32(my_chain + tp.tid + kGemmThreads * p) : 0.0f;
-#pragma unroll
-            for (int p = 0; p < kChainPerThread; ++p) lds[tp.tid + kGemmThreads * p] = in[p];
+                store_shared_f32(my_chain + tp.tid + kGemmThreads * p, lds[tp.tid + kGemmThreads * p]);
+            stores_done();
+            __syncthreads();
         }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < Cfg::kTilesM; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = tp.wm0 + 32 * i + 8 * (r / 4) + 4 * tp.half + (r % 4);
-#pragma unroll
-                for (int j = 0; j < Cfg::kTilesN; ++j) {
-                    const int gi = (tp.wn0 + 32 * j + tp.l32) >> 2;
-                    float* slot = lds + row * kGroupsPerTile + gi;  // owned by this lane's quad
-                    float c = *slot;
-                    const float sq = acc[i][j][r] * acc[i][j][r];
-                    c = c + quad_lane<0>(sq);  // element order inside the group
-                    c = c + quad_lane<1>(sq);
-                    c = c + quad_lane<2>(sq);
-                    c = c + quad_lane<3>(sq);
-                    if (kq == 0) *slot = c;
-                }
-            }
-        __syncthreads();
-#pragma unroll
-        for (int p = 0; p < kChainPerThread; ++p)
-            store_shared_f32(my_chain + tp.tid + kGemmThreads * p, lds[tp.tid + kGemmThreads * p]);
-        stores_done();
-        __syncthreads();
-        if (tp.tid == 0) __hip_atomic_store(flags + parity, step + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-        // ---- row statistics once both hand-off sequences have reached the strip's end ----
         const int n_even = (a.tiles_per_strip + 1) >> 1, n_odd = a.tiles_per_strip >> 1;
+        if (tp.tid == 0) {
+            __hip_atomic_store(&control->published[parity], step + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the tile that ends its sequence counts it; the one that ends the second commits the strip
+            if (step + 1 == (parity ? n_odd : n_even)) {
+                __builtin_amdgcn_s_waitcnt(0);
+                const int done = __hip_atomic_fetch_add(&control->sequences_done, 1, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT) + 1;
+                if (done == (n_odd > 0 ? 2 : 1)) cas_relaxed(&control->decision, 0, 1);
+            }
+        }
+
+        // ---- wait for the strip's decision ---------------------------------------------
         park_accumulators(acc);
         tp = fresh_tile_pos();
         lane = tp.tid & 63, wave = tp.tid >> 6;
-        if (!wait_for(a, flags + 0, n_even, e)) return;
-        if (n_odd > 0 && !wait_for(a, flags + 1, n_odd, e)) return;
+        bool committed = wait_for<true>(a, &control->decision, 0, e);
+        if (tp.tid == 0) {
+            int d = committed ? load_relaxed(&control->decision) : give_up(a, control);
+            if (d < 0 && committed) give_up(a, control);  // aborted by another tile: count this launch as failed
+            e.ok = d > 0 ? 1 : 0;
+        }
+        __syncthreads();
+        committed = e.ok != 0;
+        __syncthreads();
+        if (!committed) return;
+
+        // ---- row statistics: every tile finishes the rows of its strip itself ---------------
         {
             // wave w finishes rows 32 w .. 32 w + 31: lane l holds chain l of the row
             constexpr int kRowsPerWave = kTile / 4;
-            const float* mine = chain + (lane >> 5) * (kTile * kGroupsPerTile) + (lane & 31);
             const bool have = lane < 32 || n_odd > 0;
-            float part[kRowsPerWave];
 #pragma unroll
-            for (int rr = 0; rr < kRowsPerWave; ++rr)
-                part[rr] = have ? load_shared_f32(mine + (wave * kRowsPerWave + rr) * kGroupsPerTile) : 0.0f;
+            for (int set = 0; set < (WITH_GS ? 2 : 1); ++set) {
+                const float* mine = chain + set * kChainSetFloats + (lane >> 5) * (kTile * kGroupsPerTile) + (lane & 31);
+                float part[kRowsPerWave];
 #pragma unroll
-            for (int rr = 0; rr < kRowsPerWave; ++rr) {
-                const float sum_sq = tree_sum(part[rr], lane);
-                if (lane == 0) e.dn[wave * kRowsPerWave + rr] = sum_sq;  // parked; replaced below
+                for (int rr = 0; rr < kRowsPerWave; ++rr)
+                    part[rr] = have ? load_shared_f32(mine + (wave * kRowsPerWave + rr) * kGroupsPerTile) : 0.0f;
+#pragma unroll
+                for (int rr = 0; rr < kRowsPerWave; ++rr) {
+                    const float sum = tree_sum(part[rr], lane);
+                    if (lane == 0) (set == 0 ? e.dn : e.k)[wave * kRowsPerWave + rr] = sum;  // parked; replaced below
+                }
             }
         }
         __syncthreads();
         if (tp.tid < kTile) {
-            const RowStats rs = finish_row_stats(e.dn[tp.tid], 0.0f, v_old, s_old, a.in_features, 0.0f, a.rms_beta,
-                                                 a.rms_eps);
+            const RowStats rs = finish_row_stats(e.dn[tp.tid], WITH_GS ? e.k[tp.tid] : 0.0f, v_old, s_old, a.in_features,
+                                                 WITH_GS ? a.lr_scale : 0.0f, a.rms_beta, a.rms_eps);
             e.dn[tp.tid] = rs.denom;
             e.k[tp.tid] = a.cd.Cf / rs.scale_new;
             e.ratio[tp.tid] = s_old / rs.scale_new;
@@ -328,11 +425,8 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         tc.lim_pos = (float)a.geom.lim_pos;
         tc.two_m24 = 1.0f / 16777216.0f;
         tc.seed_mix = seed_mix(a.seed);
-        // 32-bit byte offsets from the state base (the launch checks that the state is smaller
-        // than 2 GiB): one add per element on top of a per-thread part
-        const uint32_t row_bytes = 3u * (uint32_t)groups_per_row;
-        const uint32_t my_state = (uint32_t)(m0 + tp.wm0 + 4 * tp.half) * row_bytes +
-                                  3u * ((uint32_t)(n0 + tp.wn0 + tp.l32) >> 2);
+        const uint32_t my_state2 = (uint32_t)(m0 + tp.wm0 + 4 * tp.half) * row_bytes +
+                                   3u * ((uint32_t)(n0 + tp.wn0 + tp.l32) >> 2);
         const uint32_t my_elem = (uint32_t)(m0 + tp.wm0 + 4 * tp.half) * (uint32_t)a.in_features +
                                  (uint32_t)(n0 + tp.wn0 + tp.l32);
         const int my_row = tp.wm0 + 4 * tp.half;
@@ -340,13 +434,11 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         for (int i = 0; i < Cfg::kTilesM; ++i)
 #pragma unroll
             for (int j = 0; j < Cfg::kTilesN; ++j) {
-                // one 4-byte load per lane and element, all 16 issued before the first tick; the
-                // tensor's last group has no byte after it, so it is fetched one byte early and
-                // shifted down
+                // all 16 state loads are issued before the first tick
                 uint32_t word[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const uint32_t off = my_state + (uint32_t)(32 * i + 8 * (r / 4) + (r % 4)) * row_bytes + 24u * j;
+                    const uint32_t off = my_state2 + (uint32_t)(32 * i + 8 * (r / 4) + (r % 4)) * row_bytes + 24u * j;
                     const uint32_t is_last = off == last_group_off ? 1u : 0u;
                     __builtin_memcpy(&word[r], a.state + (off - is_last), 4);
                     word[r] >>= 8 * is_last;
@@ -359,7 +451,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
                     const RebasedCounter c_reb{e.c_f, e.ratio[row]};
                     const uint32_t dr = (uint32_t)(32 * i + 8 * (r / 4) + (r % 4));
                     const uint32_t elem = my_elem + dr * (uint32_t)a.in_features + 32u * j;
-                    const uint32_t off = my_state + dr * row_bytes + 24u * j;
+                    const uint32_t off = my_state2 + dr * row_bytes + 24u * j;
                     const uint32_t code = (word[r] >> (6 * kq)) & 0x3fu;
                     const uint32_t nc = tick_code<false>(code, acc[i][j][r], tc, hash_first(elem), c_reb, e.q_off,
                                                          e.fin);
@@ -377,9 +469,43 @@ __global__ void strip_clear_kernel(int* words, int n) {
     if (i < n) words[i] = 0;
 }
 
-constexpr size_t kHeaderBytes = 256;  // status word, padded
+constexpr size_t kHeaderBytes = 256;  // launch-local status word, padded
 
-size_t flags_bytes(size_t strips) { return (strips * 2 * sizeof(int) + 255) / 256 * 256; }
+size_t control_bytes(size_t strips) { return (strips * sizeof(StripControl) + 255) / 256 * 256; }
+
+// Workgroups of strip launches that gave up since the last mcc_compact_counter_fused_check, one
+// counter per GPU.  It lives in the library, not in the caller's workspace: workspaces are shared
+// between layers, and the next layer's step would wipe a status word kept there.
+static __device__ int g_failures;
+
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+    int* failures = nullptr;          // device address of g_failures on this device
+    hipEvent_t last_launch = nullptr; // recorded after the most recent strip launch
+    hipStream_t last_stream = nullptr;
+    bool launched = false;
+};
+std::mutex g_mu;
+DeviceState g_devices[kMaxDevices];
+
+// The calling thread's current device with its state resolved (nullptr + *err on failure).
+DeviceState* current_device_state(hipError_t* err) {
+    int device = -1;
+    *err = hipGetDevice(&device);
+    if (*err != hipSuccess) return nullptr;
+    if (device < 0 || device >= kMaxDevices) {
+        *err = hipErrorInvalidDevice;
+        return nullptr;
+    }
+    DeviceState& d = g_devices[device];
+    if (!d.failures) {
+        void* p = nullptr;
+        *err = hipGetSymbolAddress(&p, HIP_SYMBOL(g_failures));
+        if (*err != hipSuccess) return nullptr;
+        d.failures = static_cast<int*>(p);
+    }
+    return &d;
+}
 
 }  // namespace
 
@@ -399,12 +525,25 @@ bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch)
 size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch) {
     if (!fused_strip_supports(in_features, out_features, batch)) return 0;
     const size_t strips = out_features / kTile;
-    return kHeaderBytes + flags_bytes(strips) + strips * kStripChainFloats * sizeof(float);
+    return kHeaderBytes + control_bytes(strips) + strips * kStripChainFloats * sizeof(float);
+}
+
+hipError_t fused_strip_take_failures(int* count) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    hipError_t err;
+    DeviceState* d = current_device_state(&err);
+    if (!d) return err;
+    err = hipMemcpy(count, d->failures, sizeof(int), hipMemcpyDeviceToHost);
+    if (err != hipSuccess || *count == 0) return err;
+    const int zero = 0;
+    return hipMemcpy(d->failures, &zero, sizeof(int), hipMemcpyHostToDevice);
 }
 
 hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, float* v, const float* grad_out,
                               const float* x, void* workspace, int C, int in_features, int out_features, int tokens,
-                              float lr, float rms_beta, float rms_eps, uint32_t seed, unsigned spin_limit) {
+                              float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed,
+                              unsigned spin_limit, bool* busy) {
+    *busy = false;
     const int strips = out_features / kTile;
     StripArgs a;
     a.state = state;
@@ -414,8 +553,8 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     a.x = x;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     a.status = reinterpret_cast<int*>(ws);
-    a.flags = reinterpret_cast<int*>(ws + kHeaderBytes);
-    a.chain = reinterpret_cast<float*>(ws + kHeaderBytes + flags_bytes((size_t)strips));
+    a.control = reinterpret_cast<StripControl*>(ws + kHeaderBytes);
+    a.chain = reinterpret_cast<float*>(ws + kHeaderBytes + control_bytes((size_t)strips));
     a.tokens = tokens;
     a.in_features = in_features;
     a.out_features = out_features;
@@ -425,6 +564,7 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     a.cd = make_codec(C);
     a.geom = lut_geom(a.cd);
     a.lr = lr;
+    a.lr_scale = lr_scale;
     a.rms_beta = rms_beta;
     a.rms_eps = rms_eps;
     a.seed = seed;
@@ -433,13 +573,35 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     if ((reinterpret_cast<uintptr_t>(x) & 15u) != 0) return hipErrorInvalidValue;
     // measured: with the rotating priority the direct-to-LDS main loop is 2 % slower here (it is
     // 3 % faster in the plain contraction), so the staged loop stays
-    const bool direct = false;
-    auto kernel = direct ? fused_strip_kernel<true, true>
-                         : (vec_a ? fused_strip_kernel<true, false> : fused_strip_kernel<false, false>);
+    const bool gs = lr_scale != 0.0f;
+    auto kernel = vec_a ? (gs ? fused_strip_kernel<true, false, true> : fused_strip_kernel<true, false, false>)
+                        : (gs ? fused_strip_kernel<false, false, true> : fused_strip_kernel<false, false, false>);
+
+    std::lock_guard<std::mutex> lock(g_mu);
+    hipError_t err;
+    DeviceState* dev = current_device_state(&err);
+    if (!dev) return err;
+    a.failures = dev->failures;
+
+    // Tiles of a strip wait for each other, so every workgroup of the launch has to be resident:
+    // a second strip launch running beside this one on another stream could starve both.  Refuse
+    // it (the caller orders the two).  A stream under capture is left alone: what its graph later
+    // runs beside is the caller's to order.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
+    const bool capturing = capture != hipStreamCaptureStatusNone;
+    if (!capturing && dev->launched && dev->last_stream != stream) {
+        const hipError_t q = hipEventQuery(dev->last_launch);
+        (void)hipGetLastError();  // "not ready" is an answer here, not a failure to carry along
+        if (q == hipErrorNotReady) {
+            *busy = true;
+            return hipSuccess;
+        }
+    }
 
     // the whole grid must be resident at once: size it from what the device can hold
     int device = 0, cus = 0, per_cu = 0;
-    hipError_t err = hipGetDevice(&device);
+    err = hipGetDevice(&device);
     if (err != hipSuccess) return err;
     err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
     if (err != hipSuccess) return err;
@@ -453,13 +615,23 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     const long whole = capacity / a.tiles_per_strip * a.tiles_per_strip;
     const int grid = (int)(whole < a.total_tiles ? whole : a.total_tiles);
 
-    const int clear_words = (int)((kHeaderBytes + flags_bytes((size_t)strips)) / sizeof(int));
+    const int clear_words = (int)((kHeaderBytes + control_bytes((size_t)strips)) / sizeof(int));
     hipLaunchKernelGGL(strip_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, stream,
                        reinterpret_cast<int*>(ws), clear_words);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kGemmThreads), 0, stream, a);
-    return hipGetLastError();
+    err = hipGetLastError();
+    if (err != hipSuccess || capturing) return err;
+    if (!dev->last_launch) {
+        err = hipEventCreateWithFlags(&dev->last_launch, hipEventDisableTiming);
+        if (err != hipSuccess) return err;
+    }
+    err = hipEventRecord(dev->last_launch, stream);
+    if (err != hipSuccess) return err;
+    dev->last_stream = stream;
+    dev->launched = true;
+    return hipSuccess;
 }
 
 }  // namespace mcc

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_edge_ke
         for (int p = 0; p < 4; ++p) {
             const int idx = tid + kGemmThreads * p;
             const int row = idx >> 3, c4 = idx & 7;
-            float4 x = load4<VEC_A>(a.act, m0 + row, k0 + 4 * c4, a.rows, K);
+            float4 x = load4<VEC_A>(a.act, m0 + row, k0 + 4 * c4, a.rows, K, K);
             if (!FORWARD) {  // (grad_out * scale) first, as the reference does
                 const int o = k0 + 4 * c4;
                 x.x = x.x * (o + 0 < K ? a.scale[o + 0] : 0.0f);

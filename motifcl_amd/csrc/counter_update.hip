@@ -241,7 +241,7 @@ __device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, i
     const int g_end = group_end < gpr ? group_end : gpr;
     const float* g_row = t.grad_w + (size_t)row * t.in_features;
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
-    const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
+    const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
     for (int gi = group_begin + lane; gi < g_end; gi += kWave) {
         float g[4];
 #pragma unroll
@@ -316,7 +316,7 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
         apply_streamed(t, row, lane, rc.tc, luts);
         return;
     }
-    const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
+    const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const uint32_t gi = (uint32_t)lane + kWave * j;
@@ -402,7 +402,7 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
         apply_streamed(t, row, lane, rc.tc, luts);
         return;
     }
-    const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
+    const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
     for (int c0 = 0; c0 < iters; c0 += kChunk) {
         float4 q[kChunk];
         uint32_t w[kChunk];
@@ -615,7 +615,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
             apply_streamed(t, row, lane, tc, sh.luts, j0 * kWave, (j0 + J) * kWave);
             continue;
         }
-        const uint32_t row_elem = (uint32_t)row * (uint32_t)t.in_features;
+        const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
 #pragma unroll
         for (int jj = 0; jj < J; ++jj) {
             if (j0 + jj < iters) {  // wave-uniform
@@ -817,11 +817,11 @@ hipError_t launch_update_batch(hipStream_t stream, const UpdateTensor* tensors, 
 hipError_t launch_update_dense(hipStream_t stream, uint8_t* state, float* scale, float* v,
                                const float* grad_w, int C, int in_features, int out_features,
                                float lr, float lr_scale, float rms_beta, float rms_eps,
-                               uint32_t seed) {
+                               uint32_t seed, int first_row) {
     UpdateTensor t;
     t.state = state; t.scale = scale; t.v = v; t.grad_w = grad_w;
     t.in_features = in_features; t.out_features = out_features;
-    t.row_start = 0; t.seed = seed; t.lr = lr; t.pad = 0;
+    t.row_start = 0; t.seed = seed; t.lr = lr; t.first_row = first_row;
     return launch_update_batch(stream, &t, 1, C, lr_scale, rms_beta, rms_eps);
 }
 

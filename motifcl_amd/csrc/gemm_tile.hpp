@@ -35,12 +35,13 @@ struct TileCfg {
     static constexpr int kLdsFloats = kBK * (kLdA + kLdB);
 };
 
-// One slab row segment of 4 floats, zero-filled outside the matrix.
+// One slab row segment of 4 floats, zero-filled outside the matrix (`rows` x `cols`, rows
+// `stride` floats apart).
 template <bool VEC>
-__device__ __forceinline__ float4 load4(const float* __restrict__ base, int row, int col, int rows, int cols) {
+__device__ __forceinline__ float4 load4(const float* __restrict__ base, int row, int col, int rows, int cols, int stride) {
     float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
     if (row >= rows) return r;
-    const float* p = base + (size_t)row * cols + col;
+    const float* p = base + (size_t)row * stride + col;
     if (VEC) {
         if (col + 3 < cols) return *reinterpret_cast<const float4*>(p);
     }
@@ -96,7 +97,8 @@ __device__ __forceinline__ TileXY xcd_tile(int tiles_x, int tiles_y, int band_ro
 }
 
 // Accumulates the BM x BN tile at (m0, n0) over all K tokens into acc (zeroed here).  lds holds
-// TileCfg::kLdsFloats floats.  Ends with a barrier, so lds may be reused right after.
+// TileCfg::kLdsFloats floats.  Ends with a barrier, so lds may be reused right after.  `a` is
+// K x M with rows `lda` floats apart (lda > M when a is a column band of a wider matrix).
 // Accumulator layout (v_mfma_f32_32x32x2_f32): acc[i][j][r] is row
 // wm0 + 32 i + 8 (r/4) + 4 half + r%4 and column wn0 + 32 j + l32 of the tile.
 //
@@ -121,7 +123,7 @@ __device__ __forceinline__ void gemm_tile_mainloop(const float* __restrict__ a, 
                                                    int K, int M, int N, int m0, int n0, const TilePos& tp,
                                                    float* lds,
                                                    floatx16 (&acc)[TileCfg<BM, BN>::kTilesM][TileCfg<BM, BN>::kTilesN],
-                                                   int priority_phase = 0) {
+                                                   int lda, int priority_phase = 0) {
     using Cfg = TileCfg<BM, BN>;
     float* lds_a = lds;
     float* lds_b = lds + kBK * Cfg::kLdA;
@@ -138,13 +140,13 @@ __device__ __forceinline__ void gemm_tile_mainloop(const float* __restrict__ a, 
         for (int p = 0; p < Cfg::kA4; ++p) {
             const int idx = tp.tid + kGemmThreads * p;
             const int row = idx / (BM / 4), c4 = idx % (BM / 4);
-            ra[p] = load4<VEC_A>(a, k0 + row, m0 + 4 * c4, K, M);
+            ra[p] = load4<VEC_A>(a, k0 + row, m0 + 4 * c4, K, M, lda);
         }
 #pragma unroll
         for (int p = 0; p < Cfg::kB4; ++p) {
             const int idx = tp.tid + kGemmThreads * p;
             const int row = idx / (BN / 4), c4 = idx % (BN / 4);
-            rb[p] = load4<VEC_B>(b, k0 + row, n0 + 4 * c4, K, N);
+            rb[p] = load4<VEC_B>(b, k0 + row, n0 + 4 * c4, K, N, N);
         }
     };
     auto stage = [&]() {
@@ -206,7 +208,8 @@ struct DirectCfg {
 template <int BM, int BN, bool ROTATE_PRIORITY = false>
 __device__ __forceinline__ void gemm_tile_mainloop_direct(
     const float* __restrict__ a, const float* __restrict__ b, int K, int M, int N, int m0, int n0, const TilePos& tp,
-    float* lds, floatx16 (&acc)[TileCfg<BM, BN>::kTilesM][TileCfg<BM, BN>::kTilesN], int priority_phase = 0) {
+    float* lds, floatx16 (&acc)[TileCfg<BM, BN>::kTilesM][TileCfg<BM, BN>::kTilesN], int lda,
+    int priority_phase = 0) {
     using Cfg = TileCfg<BM, BN>;
     using D = DirectCfg<BM, BN>;
 #pragma unroll
@@ -226,7 +229,7 @@ __device__ __forceinline__ void gemm_tile_mainloop_direct(
             const int chunk = p * 4 + wave;         // 64 consecutive float4 of the slab
             const int idx = chunk * 64 + lane;
             const int row = idx / (BM / 4), c4 = idx % (BM / 4);
-            __builtin_amdgcn_global_load_lds((global_ptr)(a + (size_t)(k0 + row) * M + m0 + 4 * c4),
+            __builtin_amdgcn_global_load_lds((global_ptr)(a + (size_t)(k0 + row) * lda + m0 + 4 * c4),
                                              (lds_ptr)(dst_a + chunk * 256), 16, 0, 0);
         }
 #pragma unroll

@@ -13,12 +13,12 @@ namespace mcc {
 namespace {
 
 // Token chunk blockIdx.z of `chunk` tokens goes to slice blockIdx.z of `c` (slices are m*n floats
-// apart); with one chunk this is the whole contraction.
+// apart); with one chunk this is the whole contraction.  Rows of `a` are lda floats apart.
 template <int BM, int BN, bool VEC_A, bool VEC_B, bool DIRECT>
 __global__ __launch_bounds__(kGemmThreads) void gemm_tn_kernel(const float* __restrict__ a,
                                                                 const float* __restrict__ b,
                                                                 float* __restrict__ c, int K, int M, int N,
-                                                                int chunk) {
+                                                                int chunk, int lda) {
     using Cfg = TileCfg<BM, BN>;
     __shared__ float lds[DIRECT ? DirectCfg<BM, BN>::kLdsFloats : Cfg::kLdsFloats];
     const TilePos tp = tile_pos<BM, BN>();
@@ -27,14 +27,14 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tn_kernel(const float* __re
     const int n0 = tile.x * BN;
     const int k_begin = blockIdx.z * chunk;
     const int k_len = K - k_begin < chunk ? K - k_begin : chunk;
-    a += (size_t)k_begin * M;
+    a += (size_t)k_begin * lda;
     b += (size_t)k_begin * N;
     c += (size_t)blockIdx.z * M * N;
     floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
     if (DIRECT)
-        gemm_tile_mainloop_direct<BM, BN>(a, b, k_len, M, N, m0, n0, tp, lds, acc);
+        gemm_tile_mainloop_direct<BM, BN>(a, b, k_len, M, N, m0, n0, tp, lds, acc, lda);
     else
-        gemm_tile_mainloop<BM, BN, VEC_A, VEC_B>(a, b, k_len, M, N, m0, n0, tp, lds, acc);
+        gemm_tile_mainloop<BM, BN, VEC_A, VEC_B>(a, b, k_len, M, N, m0, n0, tp, lds, acc, lda);
 #pragma unroll
     for (int i = 0; i < Cfg::kTilesM; ++i)
 #pragma unroll
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tn_group_kernel(GemmGroupAr
     const float* b = it.b + (size_t)k_begin * it.N;
     float* c = it.out + (size_t)z * it.M * it.N;
     floatx16 acc[Cfg::kTilesM][Cfg::kTilesN];
-    gemm_tile_mainloop<BM, BN, true, true>(a, b, k_len, it.M, it.N, m0, n0, tp, lds, acc);
+    gemm_tile_mainloop<BM, BN, true, true>(a, b, k_len, it.M, it.N, m0, n0, tp, lds, acc, it.M);
 #pragma unroll
     for (int ii = 0; ii < Cfg::kTilesM; ++ii)
 #pragma unroll
@@ -144,25 +144,26 @@ __global__ __launch_bounds__(256) void reduce_slices_group_kernel(ReduceGroupArg
 // the matrix: m and n stay the row lengths)
 template <int BM, int BN>
 hipError_t launch_tile(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n,
-                       const GemmTnPlan& plan, int tiles_x = 0, int tiles_y = 0) {
+                       const GemmTnPlan& plan, int tiles_x = 0, int tiles_y = 0, int lda = 0) {
+    if (lda == 0) lda = m;
     const dim3 grid(tiles_x > 0 ? tiles_x : (n + BN - 1) / BN, tiles_y > 0 ? tiles_y : (m + BM - 1) / BM, plan.splits);
     // every chunk starts at a multiple of 16 tokens, so it is as aligned as the matrix itself
-    const bool vec_a = (m % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15u) == 0);
+    const bool vec_a = (m % 4 == 0) && (lda % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15u) == 0);
     const bool vec_b = (n % 4 == 0) && ((reinterpret_cast<uintptr_t>(b) & 15u) == 0);
     // whole tiles and whole slabs (every chunk is a multiple of 16 tokens when k is): direct-to-LDS
     const bool direct = vec_a && vec_b && m % BM == 0 && n % BN == 0 && k % kBK == 0;
     if (direct)
         hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, true, true, true>), grid, dim3(kGemmThreads), 0, stream, a, b, c, k,
-                           m, n, plan.chunk);
+                           m, n, plan.chunk, lda);
     else if (vec_a && vec_b)
         hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, true, true, false>), grid, dim3(kGemmThreads), 0, stream, a, b, c,
-                           k, m, n, plan.chunk);
+                           k, m, n, plan.chunk, lda);
     else if (vec_b)
         hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, true, false>), grid, dim3(kGemmThreads), 0, stream, a, b, c,
-                           k, m, n, plan.chunk);
+                           k, m, n, plan.chunk, lda);
     else
         hipLaunchKernelGGL((gemm_tn_kernel<BM, BN, false, false, false>), grid, dim3(kGemmThreads), 0, stream, a, b,
-                           c, k, m, n, plan.chunk);
+                           c, k, m, n, plan.chunk, lda);
     return hipGetLastError();
 }
 
@@ -219,11 +220,26 @@ size_t gemm_tn_slices(int k, int m, int n) { return (size_t)plan_gemm_tn(k, m, n
 // `slices` holds plan.splits * m * n floats when the plan splits the tokens (it may start at c);
 // it is not touched otherwise.
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n,
-                              float* slices, int mode) {
-    const GemmTnPlan plan = plan_gemm_tn(k, m, n);
+                              float* slices, int mode, int lda, const GemmTnPlan* band_plan) {
+    GemmTnPlan plan = plan_gemm_tn(k, m, n);
+    if (band_plan && lda != 0 && lda != m) {
+        plan.splits = band_plan->splits;  // the tile size follows the rows at hand (a last, shorter band)
+        plan.chunk = band_plan->chunk;
+    }
     float* out = plan.splits > 1 ? slices : c;
     if (plan.splits > 1 && !slices) return hipErrorInvalidValue;
     hipError_t e;
+    if (lda != 0 && lda != m) {
+        // a column band of a wider matrix: the general tiles only
+        e = plan.tile == 128 ? launch_tile<128, 128>(stream, a, b, out, k, m, n, plan, 0, 0, lda)
+                             : launch_tile<64, 64>(stream, a, b, out, k, m, n, plan, 0, 0, lda);
+        if (e != hipSuccess || plan.splits == 1) return e;
+        const size_t mn_band = (size_t)m * n;
+        const size_t want_band = (mn_band + 255) / 256;
+        hipLaunchKernelGGL(reduce_slices_kernel, dim3((unsigned)(want_band < 4096 ? want_band : 4096)), dim3(256), 0, stream,
+                           slices, c, mn_band, plan.splits);
+        return hipGetLastError();
+    }
     const bool wide_ok = plan.tile == 128 && gemm_tn_wide_supports(a, b, k, m, n, plan.chunk);
     // rows or columns of wide tiles that make whole rounds, when the whole matrix does not
     const int wide_rows = wide_ok && plan.splits == 1 ? wide_block(m / 256, n / 256) : 0;

@@ -30,17 +30,19 @@ struct UpdateTensor {
     int row_start;  // first row of this tensor in the launch's concatenated row space
     uint32_t seed;
     float lr;
-    int pad;
+    int first_row;  // rows 0.. of this descriptor are rows first_row.. of the tensor they belong to
+                    // (a row band updated on its own): the draw hashes the tensor's element index
 };
 constexpr int kMaxUpdateBatch = 64;  // tensors per launch: the descriptors travel as kernel arguments
 
 hipError_t launch_update_batch(hipStream_t stream, const UpdateTensor* tensors, size_t n, int C,
                                float lr_scale, float rms_beta, float rms_eps);
 
+// state, scale, v and grad_w start at row `first_row` of the tensor (0: the whole tensor)
 hipError_t launch_update_dense(hipStream_t stream, uint8_t* state, float* scale, float* v,
                                const float* grad_w, int C, int in_features, int out_features,
                                float lr, float lr_scale, float rms_beta, float rms_eps,
-                               uint32_t seed);
+                               uint32_t seed, int first_row = 0);
 
 // c[m,n] = a[k,m]^T . b[k,n].  Small outputs split the k range into plan.splits chunks whose
 // partial products go to `slices` (plan.splits * m * n floats, may start at c) and are then summed
@@ -54,8 +56,11 @@ GemmTnPlan plan_gemm_tn(int k, int m, int n);
 size_t gemm_tn_slices(int k, int m, int n);
 // mode: 0 = fp32 matrix instruction; 1 = both operands split into three bf16 terms, six bf16
 // passes (gemm_tn_bf16x6.hip), where the shape allows it
+// lda: floats between rows of a (0 = m); a wider lda contracts a column band of a [k, lda] matrix,
+// cut up as `band_plan` says (the caller sized `slices` for it) instead of by the band's own shape
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c,
-                              int k, int m, int n, float* slices, int mode = 0);
+                              int k, int m, int n, float* slices, int mode = 0, int lda = 0,
+                              const GemmTnPlan* band_plan = nullptr);
 // 256 x 256-tile form of the contraction for whole tiles (gemm_tn_f32_wide.hip)
 bool gemm_tn_wide_supports(const float* a, const float* b, int k, int m, int n, int chunk);
 hipError_t launch_gemm_tn_wide(hipStream_t stream, const float* a, const float* b, float* out, int k, int m, int n,
@@ -76,17 +81,21 @@ hipError_t launch_gemm_tn_bf16x6(hipStream_t stream, const float* a, const float
                                  int k, int m, int n, const GemmTnPlan& plan);
 
 // Fused step that keeps G in the contraction's accumulators (counter_fused_strip.hip).
-// Shapes: in_features and out_features multiples of 128; lr_scale == 0 is implied.
+// Shapes: in_features and out_features multiples of 128.
 bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch);
 size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch);
 // Polls one device-side wait of the strip step may spend before it gives up (0 restores the
 // default, about four seconds; a test aid declared in motifcl_amd_diag.h).
 unsigned fused_strip_spin_limit();
 void set_fused_strip_spin_limit(unsigned spins);
+// *busy: another strip launch of this process is still running on a different stream of the GPU
+// (nothing was enqueued).  Strip launches that give up a wait raise a per-device count that
+// fused_strip_take_failures reads and clears (the stream must have been synchronised).
 hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, float* v,
                               const float* grad_out, const float* x, void* workspace, int C,
-                              int in_features, int out_features, int tokens, float lr, float rms_beta,
-                              float rms_eps, uint32_t seed, unsigned spin_limit);
+                              int in_features, int out_features, int tokens, float lr, float lr_scale,
+                              float rms_beta, float rms_eps, uint32_t seed, unsigned spin_limit, bool* busy);
+hipError_t fused_strip_take_failures(int* count);
 
 hipError_t launch_decode_weight(hipStream_t stream, const uint8_t* state, const float* scale,
                                 float* weight, int C, int in_features, int out_features);

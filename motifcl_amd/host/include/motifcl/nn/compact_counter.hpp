@@ -12,18 +12,20 @@
 namespace motifcl::nn {
 
 // How the fused update holds the weight gradient while it needs the whole row's RMS:
-//   Strip  the gradient never leaves the contraction's registers; tiles of a 128-row strip
-//          exchange 32 KiB of partial row sums (no weight-sized buffer, as in the reference,
-//          tests/test_memory_truth_gate.cpp:109-113); needs lr_scale == 0 and in/out multiples
-//          of 128, other layers silently use Full
-//   Full   contraction into f32[out,in] workspace slices, then the update kernel (about 10 percent
-//          faster on large layers; the only way to keep the GPU busy on small ones, whose token
-//          range is split over many workgroups)
-//   Auto   Strip for layers of at least 128 tiles of 128 x 128 (2M weights), Full below
-// Strip and Full give identical bytes wherever Full does not split the tokens into chunks (fewer
-// than 512 tokens, or at least 1024 tiles); elsewhere Full adds chunk sums and the two differ by
-// that rounding, both within the tolerance the contraction is held to.
-enum class FusedWorkspace { Auto, Strip, Full };
+//   Full   contraction into f32[out,in] workspace slices, then the update kernel: the fastest way
+//          (about 10 percent on large layers; on small ones the only way to keep the GPU busy,
+//          their token range being split over many workgroups).  The default.
+//   Small  no weight-sized buffer exists at any time, as in the reference
+//          (tests/test_memory_truth_gate.cpp:109-113).  Layers of 128-multiples with rows of at
+//          least 768 weights keep the gradient in the contraction's registers and exchange 512
+//          bytes of partial row sums per output row between the tiles of a 128-row strip; every
+//          other layer is updated band by band of an eighth of its rows through a workspace of that
+//          size.  Any lr_scale.  check_fused_update() reports a strip step that gave up an
+//          inter-tile wait (such a step leaves whole 128-row strips without their update).
+// Small and Full give identical bytes wherever neither splits the tokens into chunks (fewer than
+// 512 tokens, or at least 1024 tiles of 128 x 128); elsewhere they add chunk sums in different
+// order and differ by that rounding, both within the tolerance the contraction is held to.
+enum class FusedWorkspace { Full, Small };
 
 class CounterStateLinear;
 
@@ -81,7 +83,8 @@ public:
     void set_deferred(DeferredCounterUpdates* d) { deferred_ = d; }
     DeferredCounterUpdates* deferred() const { return deferred_; }
     FusedWorkspace fused_workspace() const { return fused_workspace_; }
-    // Waits for the backend and throws if the last Strip update gave up an inter-tile wait.
+    // Waits for the backend and throws if a Small-workspace step on this GPU gave up an inter-tile
+    // wait since the last check.
     void check_fused_update() const;
     void set_lr(float lr) { lr_ = lr; }
     float lr() const { return lr_; }
@@ -105,7 +108,7 @@ private:
     float rms_eps_ = 1e-3f;
     std::uint32_t seed_ = 12345u;
     bool training_ = true;
-    FusedWorkspace fused_workspace_ = FusedWorkspace::Auto;
+    FusedWorkspace fused_workspace_ = FusedWorkspace::Full;
     DeferredCounterUpdates* deferred_ = nullptr;
     friend class DeferredCounterUpdates;
     std::size_t last_fused_ws_ = 0, last_fused_batch_ = 0;

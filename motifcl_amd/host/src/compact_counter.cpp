@@ -109,10 +109,8 @@ void CounterStateLinear::apply_update_backward(const Tensor& grad_out, const Ten
     const std::size_t N = static_cast<std::size_t>(x.shape()[0]);
     const std::size_t in = static_cast<std::size_t>(in_), out = static_cast<std::size_t>(out_);
     std::size_t ws = 0;
-    const bool large = ((in + 127) / 128) * ((out + 127) / 128) >= 128;
-    if (lr_scale_ == 0.0f && (fused_workspace_ == FusedWorkspace::Strip ||
-                              (fused_workspace_ == FusedWorkspace::Auto && large)))
-        ws = mcc_compact_counter_fused_strip_workspace_nbytes(in, out, N);  // 0: shape not supported
+    if (fused_workspace_ == FusedWorkspace::Small)
+        ws = mcc_compact_counter_fused_strip_workspace_nbytes(in, out, N);  // 0: no smaller way for this shape
     if (ws == 0) ws = mcc_compact_counter_fused_workspace_nbytes(in, out, N);
     void* scratch = backend_->workspace(ws);
     // exactly ws bytes are lent: the size selects how the step runs
@@ -173,10 +171,11 @@ void DeferredCounterUpdates::flush() {
 }
 
 void CounterStateLinear::check_fused_update() const {
-    if (last_fused_ws_ == 0) return;
-    const int rc = mcc_compact_counter_fused_check(backend_->hip_stream(), backend_->workspace(last_fused_ws_),
-                                                   last_fused_ws_, static_cast<std::size_t>(in_),
-                                                   static_cast<std::size_t>(out_), last_fused_batch_);
+    // the library counts given-up strip steps per GPU, not per workspace: the answer covers every
+    // layer's step on this GPU since the last check
+    const int rc = mcc_compact_counter_fused_check(backend_->hip_stream(), backend_->workspace(1), 1,
+                                                   static_cast<std::size_t>(in_), static_cast<std::size_t>(out_),
+                                                   last_fused_batch_ ? last_fused_batch_ : 1);
     MCL_CHECK(rc == MCC_OK, std::string("hip compact-counter fused update failed: ") + mcc_last_error());
 }
 

@@ -23,6 +23,27 @@ inline void fill_deterministic(std::vector<float>& values, std::uint32_t seed, f
     }
 }
 
+// Counter-based generator of this build: lowbias32 of the index and the stream, 24 bits to a
+// uniform in (0, 1), Box-Muller for normals.  The same values on every host and standard library
+// (std::normal_distribution and std::uniform_int_distribution are implementation-defined).
+inline std::uint32_t mix32(std::uint32_t x) {
+    x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    return x;
+}
+inline float uniform_open(std::uint32_t stream, std::uint32_t index) {
+    return (static_cast<float>(mix32(index ^ mix32(stream)) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+}
+inline float normal_at(std::uint32_t stream, std::uint32_t index) {
+    const float u1 = uniform_open(stream, 2u * index), u2 = uniform_open(stream, 2u * index + 1u);
+    return std::sqrt(-2.0f * std::log(u1)) * std::cos(6.28318530717958647692f * u2);
+}
+inline void fill_normal(std::vector<float>& values, std::uint32_t stream, float sigma) {
+    for (std::size_t i = 0; i < values.size(); ++i) values[i] = sigma * normal_at(stream, static_cast<std::uint32_t>(i));
+}
+inline int ternary_at(std::uint32_t stream, std::uint32_t index) {
+    return static_cast<int>(mix32(index ^ mix32(stream)) % 3u) - 1;
+}
+
 template <typename T>
 void require_exact(const std::vector<T>& actual, const std::vector<T>& expected, const std::string& label) {
     if (actual != expected) throw std::runtime_error(label + " exact mismatch");

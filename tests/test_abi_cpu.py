@@ -100,3 +100,45 @@ def test_storage_rejects_without_touching_the_device(L):
     assert L.mcc_device_free(None) == 0
     assert L.mcc_device_free(P) == -1
     assert L.mcc_device_bytes_current() == 0
+
+
+def _counter_tensor(state_ptr, n_in=8, n_out=2):
+    t = mlib.CounterTensor()
+    t.state, t.state_nbytes = state_ptr, n_out * (n_in // 4) * 3
+    t.scale, t.scale_nbytes, t.v, t.v_nbytes = P, n_out * 4, P, n_out * 4
+    t.grad_w, t.grad_w_nbytes = P, n_out * n_in * 4
+    t.in_features, t.out_features, t.lr, t.seed = n_in, n_out, 3e-3, 1
+    return t
+
+
+def test_batched_updates_reject_a_state_listed_twice_and_validate_every_tensor_first(L):
+    # two descriptors on one state would be updated by two sets of workgroups of the same launch
+    arr = (mlib.CounterTensor * 3)(_counter_tensor(0x1000), _counter_tensor(0x2000), _counter_tensor(0x1000))
+    assert L.mcc_compact_counter_apply_update_dense_batched(None, arr, 3, 11, 0.0, 0.9, 1e-3) == -1
+    assert "same state twice" in L.mcc_last_error().decode()
+    # an invalid tensor anywhere in the list is reported before anything is enqueued
+    arr = (mlib.CounterTensor * 2)(_counter_tensor(0x1000), _counter_tensor(0x2000, n_in=6))
+    assert L.mcc_compact_counter_apply_update_dense_batched(None, arr, 2, 11, 0.0, 0.9, 1e-3) == -1
+    assert L.mcc_last_error().decode().startswith("tensor 1:")
+
+    def fused(state_ptr, n_in=8):
+        t = mlib.FusedTensor()
+        t.state, t.state_nbytes = state_ptr, 2 * (n_in // 4) * 3
+        t.scale, t.scale_nbytes, t.v, t.v_nbytes = P, 8, P, 8
+        t.grad_out, t.grad_out_nbytes, t.x, t.x_nbytes = P, 4 * 2 * 4, P, 4 * n_in * 4
+        t.in_features, t.out_features, t.batch, t.lr, t.seed = n_in, 2, 4, 3e-3, 1
+        return t
+
+    for mode in (0, 1):  # fp32 instruction, split-bf16 contraction: the same checks before any launch
+        assert L.mcc_set_contraction_mode(mode) == 0
+        try:
+            arr = (mlib.FusedTensor * 2)(fused(0x1000), fused(0x1000))
+            need = L.mcc_compact_counter_fused_batched_workspace_nbytes(arr, 2)
+            assert L.mcc_compact_counter_apply_update_fused_batched(None, arr, 2, 0x10000, need, 11, 0.0, 0.9, 1e-3) == -1
+            assert "same state twice" in L.mcc_last_error().decode()
+            arr = (mlib.FusedTensor * 2)(fused(0x1000), fused(0x2000, n_in=6))
+            need = L.mcc_compact_counter_fused_batched_workspace_nbytes(arr, 2)
+            assert L.mcc_compact_counter_apply_update_fused_batched(None, arr, 2, 0x10000, need, 11, 0.0, 0.9, 1e-3) == -1
+            assert L.mcc_last_error().decode().startswith("tensor 1:")
+        finally:
+            L.mcc_set_contraction_mode(0)

@@ -26,7 +26,7 @@ STRIP_SHAPES = [
 ]
 
 
-def run_both(ops, n, n_in, n_out, C, seed, lr=HP["lr"]):
+def run_both(ops, n, n_in, n_out, C, seed, lr=HP["lr"], lr_scale=HP["lr_scale"]):
     _, _, _, scale, v = synth.counter_case(seed, n_out, n_in, C, oracle=None)
     rng = np.random.default_rng(seed + 1)
     hi = 3 * (2 * C - 1)
@@ -41,7 +41,7 @@ def run_both(ops, n, n_in, n_out, C, seed, lr=HP["lr"]):
         assert nbytes > 0
         d = [dev(state), dev(scale), dev(v)]
         ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
-        ops.apply_update_fused(*d, ddy, dx, ws, C, lr, HP["lr_scale"], HP["rms_beta"], HP["rms_eps"], 4242)
+        ops.apply_update_fused(*d, ddy, dx, ws, C, lr, lr_scale, HP["rms_beta"], HP["rms_eps"], 4242)
         ops.fused_check(ws, n_in, n_out, n)
         out.append([host(t) for t in d])
     return state, scale, v, x, dy, out
@@ -89,19 +89,100 @@ def test_strip_path_against_oracle(ops, oracle):
     assert np.array_equal(strip[1], e_scale)
 
 
-def test_strip_workspace_rules(ops):
-    assert ops.fused_strip_workspace_nbytes(288, 288, 64) == 0      # not multiples of 128
-    assert ops.fused_strip_workspace_nbytes(128, 64, 64) == 0
-    n, n_in, n_out, C = 64, 256, 128, 11
+@pytest.mark.parametrize("shape", [(64, 768, 256, 11), (96, 1024, 384, 3), (32, 4096, 4096, 11), (32, 11008, 4096, 11)],
+                         ids=lambda s: "N%d_in%d_out%d_C%d" % s)
+def test_strip_path_with_scale_learning_matches_two_kernel_path(ops, oracle, shape):
+    # lr_scale != 0: the row sums of g * t travel through the strip beside the sums of squares
+    n, n_in, n_out, C = shape
+    state, scale, v, x, dy, (full, strip) = run_both(ops, n, n_in, n_out, C, seed=n_in + n_out + 1, lr_scale=0.05)
+    assert not np.array_equal(full[1], scale)  # the scale moved
+    for a, b in zip(strip, full):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    if n_in * n_out <= 1 << 20:
+        g = host(ops.matmul_transpose_a(dev(dy), dev(x)))
+        exp = oracle.update_dense(state, scale, v, g, C, HP["lr"], 0.05, HP["rms_beta"], HP["rms_eps"], 4242)
+        for a, b in zip(strip, exp):
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+# (N, in, out, C): layers too small or too oddly shaped for the strips run band by band
+BANDED_SHAPES = [(64, 256, 256, 11),   # tests/test_memory_truth_gate.cpp:34
+                 (64, 288, 288, 11), (300, 260, 35, 3), (37, 68, 35, 3), (8, 64, 40, 3), (128, 512, 1000, 11)]
+
+
+@pytest.mark.parametrize("shape", BANDED_SHAPES, ids=lambda s: "N%d_in%d_out%d_C%d" % s)
+@pytest.mark.parametrize("lr_scale", [0.0, 0.05])
+def test_banded_small_workspace_matches_two_kernel_path(ops, oracle, shape, lr_scale):
+    # under 512 tokens neither way splits the tokens: the gradients are the same bits and so is the state
+    n, n_in, n_out, C = shape
+    small, full_n = ops.fused_strip_workspace_nbytes(n_in, n_out, n), ops.fused_workspace_nbytes(n_in, n_out, n)
+    assert 0 < small < full_n
+    if n_out >= 20:
+        assert small < n_in * n_out  # a quarter of the dense gradient (tests/test_memory_truth_gate.cpp:109-113)
+    state, scale, v, x, dy, (full, banded) = run_both(ops, n, n_in, n_out, C, seed=n_in + 7, lr_scale=lr_scale)
+    assert not np.array_equal(full[0], state)
+    for a, b in zip(banded, full):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    g = host(ops.matmul_transpose_a(dev(dy), dev(x)))
+    exp = oracle.update_dense(state, scale, v, g, C, HP["lr"], lr_scale, HP["rms_beta"], HP["rms_eps"], 4242)
+    for a, b in zip(banded, exp):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def test_banded_small_workspace_with_token_chunks_differs_only_by_rounding(ops, oracle):
+    # BASELINE config 0: 4096 tokens are contracted in chunks, differently cut for a band than for
+    # the whole layer; same terms, another order
+    n, n_in, n_out, C = 4096, 288, 288, 11
+    state, scale, v, x, dy, (full, banded) = run_both(ops, n, n_in, n_out, C, seed=3, lr_scale=0.05)
+    np.testing.assert_allclose(banded[2], full[2], rtol=1e-5)
+    np.testing.assert_allclose(banded[1], full[1], rtol=1e-4)  # the sum of g * t cancels: a few more ulps
+    assert (banded[0] != full[0]).mean() < 1e-3
+    e_state = oracle.update_fused(state, scale, v, dy, x, C, HP["lr"], 0.05, HP["rms_beta"], HP["rms_eps"], 4242)[0]
+    flips = np.mean(oracle.unpack_codes(banded[0]) != oracle.unpack_codes(e_state))
+    print("banded vs oracle: counter-flip mismatch %.3e" % flips)
+    assert flips <= 2e-3
+
+
+def test_small_workspace_rules(ops):
+    assert ops.fused_strip_workspace_nbytes(128, 64, 64) > 0        # banded
+    assert ops.fused_strip_workspace_nbytes(6, 64, 64) == 0         # in_features not a multiple of 4
+    n, n_in, n_out, C = 64, 1024, 128, 11
     _, _, _, scale, v = synth.counter_case(1, n_out, n_in, C)
     state = np.zeros(n_out * n_in // 4 * 3, dtype=np.uint8)
     x, dy = synth.activations(2, n, n_in, n_out)
     ws = torch.empty(ops.fused_strip_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
     from motifcl_amd.lib import MccError
-    with pytest.raises(MccError, match="lr_scale"):
-        ops.apply_update_fused(dev(state), dev(scale), dev(v), dev(dy), dev(x), ws, C, 3e-3, 0.05, 0.9, 1e-3, 1)
     with pytest.raises(MccError, match="too small"):
         ops.apply_update_fused(dev(state), dev(scale), dev(v), dev(dy), dev(x), ws[:-16], C, 3e-3, 0.0, 0.9, 1e-3, 1)
+
+
+def test_second_strip_step_on_another_stream_is_refused_while_the_first_runs(ops):
+    # tiles of a strip wait for each other on the device, so two such launches must not share the GPU
+    from motifcl_amd.lib import MccError
+    n, n_in, n_out, C = 8192, 4096, 4096, 11
+    rng = np.random.default_rng(0)
+    state = dev(rng.integers(0, 63, n_out * n_in // 4 * 3).astype(np.uint8))
+    state2 = state.clone()
+    scale = torch.full((n_out,), 0.02, device="cuda")
+    v = torch.zeros(n_out, device="cuda")
+    x = torch.randn(n, n_in, device="cuda")
+    dy = torch.randn(n, n_out, device="cuda") * 0.01
+    nbytes = ops.fused_strip_workspace_nbytes(n_in, n_out, n)
+    ws1 = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    ws2 = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    ops.apply_update_fused(state, scale, v, dy, x, ws1, C, 3e-3, 0.0, 0.9, 1e-3, 1)  # about 1.5 ms of work
+    with torch.cuda.stream(side):
+        with pytest.raises(MccError, match="different stream"):
+            ops.apply_update_fused(state2, scale.clone(), v.clone(), dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
+    torch.cuda.synchronize()
+    ops.fused_check(ws1, n_in, n_out, n)
+    # once the first has finished the other stream may go
+    with torch.cuda.stream(side):
+        ops.apply_update_fused(state2, scale.clone(), v.clone(), dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
+    torch.cuda.synchronize()
+    ops.fused_check(ws2, n_in, n_out, n)
 
 
 def test_two_strip_updates_in_a_row_are_deterministic(ops):
@@ -123,37 +204,53 @@ def test_two_strip_updates_in_a_row_are_deterministic(ops):
         assert np.array_equal(a, b)
 
 
-def test_given_up_wait_is_reported_and_every_workgroup_exits(ops):
-    # a spin budget of one poll makes waits fail from the host side; the kernel must still
-    # drain and the failure must surface through fused_check
+def test_given_up_wait_is_reported_and_leaves_whole_strips_untouched(ops):
+    # a spin budget of one poll makes waits fail from the host side; the kernel must still drain,
+    # the failure must surface through fused_check -- also after another layer has used the same
+    # workspace -- and every 128-row strip must be either fully updated or untouched
     import motifcl_amd
     from motifcl_amd.lib import MccError
     L = motifcl_amd.load()
-    n, n_in, n_out, C = 32, 4096, 256, 11
-    state = np.zeros(n_out * n_in // 4 * 3, dtype=np.uint8)
+    n, n_in, n_out, C = 32, 4096, 512, 11
+    rng = np.random.default_rng(4)
+    state = rng.integers(0, 63, n_out * n_in // 4 * 3).astype(np.uint8)
     scale = np.full(n_out, 0.05, dtype=F)
     v = np.zeros(n_out, dtype=F)
     x, dy = synth.activations(3, n, n_in, n_out)
     ws = torch.empty(ops.fused_strip_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
+    ref = [dev(state), dev(scale), dev(v)]
+    full = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
+    ops.apply_update_fused(*ref, dev(dy), dev(x), full, C, 3e-3, 0.0, 0.9, 1e-3, 5)
+    ref = [host(t) for t in ref]
     L.mcc_compact_counter_fused_strip_set_spin_limit(1)
     try:
         d = [dev(state), dev(scale), dev(v)]
         ops.apply_update_fused(*d, dev(dy), dev(x), ws, C, 3e-3, 0.0, 0.9, 1e-3, 5)
-        try:
-            ops.fused_check(ws, n_in, n_out, n)
-            gave_up = False
-        except MccError as err:
-            assert "gave up waiting" in str(err)
-            gave_up = True
+        torch.cuda.synchronize()
     finally:
         L.mcc_compact_counter_fused_strip_set_spin_limit(0)
-    print("wait given up with a one-poll budget:", gave_up)
+    # a second layer's step (two-kernel path) through memory that overlaps the first one's workspace
+    other = [dev(state[:256 * 256 // 4 * 3]), dev(scale[:256]), dev(v[:256])]
+    ops.apply_update_fused(*other, dev(dy[:, :256]), dev(x[:, :256]), full, 11, 3e-3, 0.0, 0.9, 1e-3, 6)
+    with pytest.raises(MccError, match="gave up waiting"):
+        ops.fused_check(ws, n_in, n_out, n)
+    ops.fused_check(ws, n_in, n_out, n)  # reported once
+    got = [host(t) for t in d]
+    row_bytes = n_in // 4 * 3
+    untouched = 0
+    for s0 in range(0, n_out, 128):
+        rows = slice(s0, s0 + 128)
+        st = slice(s0 * row_bytes, (s0 + 128) * row_bytes)
+        if np.array_equal(got[0][st], state[st]):
+            untouched += 1
+            assert np.array_equal(got[1][rows], scale[rows]) and np.array_equal(got[2][rows], v[rows])
+        else:
+            assert np.array_equal(got[0][st], ref[0][st]), "strip %d is half-updated" % (s0 // 128)
+            assert np.array_equal(got[1][rows], ref[1][rows]) and np.array_equal(got[2][rows], ref[2][rows])
+    assert untouched >= 1
     # with the default budget the same call completes and matches the two-kernel path
-    ref = [dev(state), dev(scale), dev(v)]
-    full = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
-    ops.apply_update_fused(*ref, dev(dy), dev(x), full, C, 3e-3, 0.0, 0.9, 1e-3, 5)
     d = [dev(state), dev(scale), dev(v)]
     ops.apply_update_fused(*d, dev(dy), dev(x), ws, C, 3e-3, 0.0, 0.9, 1e-3, 5)
     ops.fused_check(ws, n_in, n_out, n)
     for a, b in zip(d, ref):
-        assert torch.equal(a, b)
+        assert np.array_equal(host(a), b)

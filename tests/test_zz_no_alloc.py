@@ -71,11 +71,13 @@ def test_static_workspace_matches_lent_workspace_twice_in_a_row(ops, oracle):
 
 def test_static_workspace_takes_the_strip_path_for_large_layers(ops, oracle):
     C = 11
-    # 4096 x 4096 needs 64 MiB of full workspace: beyond the array, so the strip path runs; then a
-    # smaller strip-path-only... no: a smaller full-workspace tensor through the same array
+    # 4096 x 4096 needs 64 MiB of full workspace: beyond the array, so the strip path runs (with and
+    # without scale learning); then a smaller full-workspace tensor through the same array
     N, n_in, n_out = 64, 4096, 4096
     assert ops.fused_workspace_nbytes(n_in, n_out, N) > ops.NOALLOC_WORKSPACE_NBYTES
     case = _case(oracle, 200, N, n_in, n_out, C)
+    exp_s = _lent(ops, case, N, n_in, n_out, C, (3e-3, 0.02), 10, strip=True)
+    _same(_static(ops, case, C, (3e-3, 0.02), 10), exp_s)
     exp = _lent(ops, case, N, n_in, n_out, C, (3e-3, 0.0), 11, strip=True)
     _same(_static(ops, case, C, (3e-3, 0.0), 11), exp)
     case2 = _case(oracle, 201, 128, 1024, 512, C)
@@ -90,13 +92,20 @@ def test_static_workspace_takes_the_strip_path_for_large_layers(ops, oracle):
 
 def test_static_workspace_rejects_what_does_not_fit(ops, oracle):
     from motifcl_amd import lib as mlib
-    # 4096 x 4096 with lr_scale != 0 has no strip path and 64 MiB of full workspace
-    case = _case(oracle, 300, 16, 4096, 4096, 11)
+    # 8200 x 8200 is no multiple of 128: its smaller workspace is an eighth of 269 MB, beyond the array
+    n, n_in, n_out = 16, 8200, 8200
+    assert ops.fused_strip_workspace_nbytes(n_in, n_out, n) > ops.NOALLOC_WORKSPACE_NBYTES
+    state = torch.zeros(n_out * n_in // 4 * 3, dtype=torch.uint8, device="cuda")
+    scale = torch.full((n_out,), 0.02, device="cuda")
+    v = torch.zeros(n_out, device="cuda")
+    dy = torch.randn(n, n_out, device="cuda") * 0.01
+    x = torch.randn(n, n_in, device="cuda")
     with pytest.raises(mlib.MccError) as e:
-        _static(ops, case, 11, (3e-3, 0.01), 1)
-    assert e.value.code == -1
-    # a shape with neither: 4104 x 4096 (not a multiple of 128) at 67 MB
-    case = _case(oracle, 301, 16, 4104, 4096, 11)
-    with pytest.raises(mlib.MccError) as e:
-        _static(ops, case, 11, (3e-3, 0.0), 1)
+        ops.apply_update_fused_static(state, scale, v, dy, x, 11, 3e-3, 0.0, 0.9, 1e-3, 1)
     assert e.value.code == -1 and "static" in e.value.message
+    torch.cuda.synchronize()
+    assert int(state.max()) == 0  # nothing was enqueued
+    # invalid arguments are reported as by the lent-workspace entry point
+    with pytest.raises(mlib.MccError, match="divisible by 4"):
+        ops.apply_update_fused_static(state, scale, v, dy[:, :6].contiguous(), x[:, :6].contiguous(), 11, 3e-3, 0.0, 0.9,
+                                      1e-3, 1)
