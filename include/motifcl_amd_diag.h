@@ -3,9 +3,9 @@
  *
  * Nothing here has a counterpart in the reference and nothing here is part of
  * the drop-in boundary (that is motifcl_amd.h): a shader-clock probe used by
- * the benchmark to report the clock the kernels ran at, and the knob that lets
- * a test force the bounded device-side wait of the strip-workspace fused step
- * to give up.  Conventions (status codes, mcc_last_error) are those of
+ * the benchmark to report the clock the kernels ran at, the generator of the
+ * benchmark's synthetic inputs, and the knob that lets a test force the bounded
+ * device-side wait of the strip-workspace fused step to give up.  Conventions (status codes, mcc_last_error) are those of
  * motifcl_amd.h.
  */
 #ifndef MOTIFCL_AMD_DIAG_H
@@ -36,6 +36,20 @@ void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
  */
 int mcc_clock_probe(void* stream, uint64_t* out, size_t out_nbytes, double seconds);
 int mcc_wall_clock_khz(int* khz);
+
+/*
+ * Synthetic inputs of the benchmark, generated on the device by a counter-based generator:
+ * lowbias32 of the element index and the stream id -> two 24-bit uniforms -> Box-Muller.
+ * dst[i] = sigma * z_i for i < n.  The same (stream_id, n) gives the same bytes on every run
+ * of this library; the host copies them when the CPU needs the same inputs.
+ */
+int mcc_fill_normal_f32(void* stream, float* dst, size_t n, uint32_t stream_id, float sigma);
+
+/*
+ * Packed counter state (four 6-bit codes per 3 bytes) with every code uniform on
+ * [0, n_codes), from the same generator.  dst holds 3 * n_groups bytes.
+ */
+int mcc_fill_counter_state_u8(void* stream, uint8_t* dst, size_t n_groups, uint32_t stream_id, uint32_t n_codes);
 
 #ifdef __cplusplus
 }

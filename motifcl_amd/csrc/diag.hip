@@ -33,9 +33,71 @@ __global__ __launch_bounds__(64) void clock_probe_kernel(unsigned long long* out
     }
 }
 
+// Synthetic inputs of the benchmark, generated where they are used.  Element i of stream s:
+// two 24-bit uniforms from lowbias32(2i ^ lowbias32(s)) and lowbias32((2i+1) ^ lowbias32(s)),
+// shifted into (0, 1), Box-Muller (cosine branch), times sigma.
+__device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
+    x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    return x;
+}
+
+__global__ __launch_bounds__(256) void fill_normal_kernel(float* dst, size_t n, uint32_t stream_hash, float sigma) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint32_t lo = (uint32_t)i, hi = (uint32_t)(i >> 32);
+        const uint32_t salt = stream_hash ^ lowbias32(hi + 0x9e3779b9u * hi);
+        const float u1 = ((float)(lowbias32((2u * lo) ^ salt) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+        const float u2 = ((float)(lowbias32((2u * lo + 1u) ^ salt) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+        dst[i] = sigma * (sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2));
+    }
+}
+
+// Packed counter state with every code uniform on [0, n_codes): group g holds codes 4g .. 4g+3.
+__global__ __launch_bounds__(256) void fill_state_kernel(uint8_t* dst, size_t n_groups, uint32_t stream_hash, uint32_t n_codes) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_groups; g += stride) {
+        uint32_t word = 0;
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint64_t e = 4 * g + k;
+            const uint32_t h = lowbias32((uint32_t)e ^ stream_hash ^ lowbias32((uint32_t)(e >> 32) * 0x85ebca6bu));
+            word |= (uint32_t)(((uint64_t)h * n_codes) >> 32) << (6 * k);
+        }
+        dst[3 * g] = (uint8_t)word;
+        dst[3 * g + 1] = (uint8_t)(word >> 8);
+        dst[3 * g + 2] = (uint8_t)(word >> 16);
+    }
+}
+
 }  // namespace
 
 extern "C" {
+
+int mcc_fill_normal_f32(void* stream, float* dst, size_t n, uint32_t stream_id, float sigma) {
+    if (n == 0) return MCC_OK;
+    if (!dst) return mcc::report_failure(MCC_E_INVALID, "fill_normal received a null pointer");
+    uint32_t h = stream_id;
+    h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+    const size_t want = (n + 255) / 256;
+    hipLaunchKernelGGL(fill_normal_kernel, dim3((unsigned)(want < 65536 ? want : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), dst, n, h, sigma);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mcc::report_hip_failure(e, "fill_normal launch failed");
+    return MCC_OK;
+}
+
+int mcc_fill_counter_state_u8(void* stream, uint8_t* dst, size_t n_groups, uint32_t stream_id, uint32_t n_codes) {
+    if (n_groups == 0) return MCC_OK;
+    if (!dst) return mcc::report_failure(MCC_E_INVALID, "fill_counter_state received a null pointer");
+    if (n_codes == 0 || n_codes > 64) return mcc::report_failure(MCC_E_INVALID, "fill_counter_state needs 1..64 codes");
+    uint32_t h = stream_id ^ 0x5bd1e995u;
+    h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+    const size_t want = (n_groups + 255) / 256;
+    hipLaunchKernelGGL(fill_state_kernel, dim3((unsigned)(want < 65536 ? want : 65536)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), dst, n_groups, h, n_codes);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return mcc::report_hip_failure(e, "fill_counter_state launch failed");
+    return MCC_OK;
+}
 
 void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins) { mcc::set_fused_strip_spin_limit(spins); }
 

@@ -59,6 +59,8 @@ DIAG_SIGNATURES = {
     "mcc_compact_counter_fused_strip_set_spin_limit": (None, [ctypes.c_uint]),
     "mcc_clock_probe": (ctypes.c_int, [_vp, _vp, _sz, ctypes.c_double]),
     "mcc_wall_clock_khz": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int)]),
+    "mcc_fill_normal_f32": (ctypes.c_int, [_vp, _vp, _sz, _u32, _f]),
+    "mcc_fill_counter_state_u8": (ctypes.c_int, [_vp, _vp, _sz, _u32, _u32]),
 }
 
 

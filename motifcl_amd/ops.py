@@ -221,6 +221,22 @@ def get_contraction_mode():
     return int(_lib.load().mcc_get_contraction_mode())
 
 
+def fill_normal(t, stream_id, sigma):
+    """t[i] = sigma * z_i from the library's counter-based generator (lowbias32 -> Box-Muller)."""
+    ptr, nbytes = _buf(t, torch.float32)
+    _lib.check(_lib.load().mcc_fill_normal_f32(_stream(), ptr, nbytes // 4, stream_id & 0xFFFFFFFF, sigma))
+    return t
+
+
+def fill_counter_state(state, stream_id, n_codes):
+    """Packed state with every code uniform on [0, n_codes), same generator."""
+    ptr, nbytes = _buf(state, torch.uint8)
+    if nbytes % 3:
+        raise ValueError("a packed state holds 3 bytes per group")
+    _lib.check(_lib.load().mcc_fill_counter_state_u8(_stream(), ptr, nbytes // 3, stream_id & 0xFFFFFFFF, n_codes))
+    return state
+
+
 class ClockProbe:
     """Shader clock while other kernels run: a one-wave kernel on a side stream sleeps for
     `seconds` of the constant-rate wall clock and counts shader cycles over the same stretch.
