@@ -229,7 +229,7 @@ FUSED_SHAPES = [  # (N, in, out, C)
     (4096, 288, 288, 11),  # BASELINE config 0
     (1024, 768, 288, 11), (1024, 288, 768, 11),
     # BASELINE config 2 (dim 768, hidden 2048): square, up and down projections
-    (512, 768, 768, 11), (2048, 768, 2048, 11), (2048, 2048, 768, 11),
+    (512, 768, 768, 11), (512, 768, 2048, 11), (512, 2048, 768, 11), (2048, 768, 2048, 11), (2048, 2048, 768, 11),
     # BASELINE config 4 (dim 4096, hidden 11008) at few tokens: one shape per tile plan of the
     # contraction (whole rounds of wide tiles; wide + small tiles split by rows, by columns)
     (64, 4096, 4096, 11), (512, 4096, 4096, 11), (32, 4096, 11008, 11), (32, 11008, 4096, 11),
