@@ -25,6 +25,18 @@ extern "C" {
 void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
 
 /*
+ * The contraction of shapes that are more than two but not a whole number of rounds of
+ * 256 x 256 tiles runs as one launch in which neighbouring workgroups hand a partly
+ * summed tile on through the output buffer; a workgroup that does not find the tile it
+ * is to continue computes it alone.  `polls` is the number of polls (about a
+ * microsecond each) before it does so (0xffffffff restores the default); a non-zero
+ * `start_first` makes every workgroup look for that tile before its neighbour can have
+ * produced it.  With (0, 1) every hand-off takes the fallback; the result is the same
+ * bits either way, which is what the test that uses this checks.
+ */
+void mcc_contraction_spans_set_test_mode(unsigned polls, int start_first);
+
+/*
  * Shader-clock probe (a measurement aid with no counterpart in the reference).
  * Enqueues a one-wave kernel on `stream` that sleeps for `seconds` (at most 2) of
  * the constant-rate wall clock and writes two 64-bit counts to the device buffer

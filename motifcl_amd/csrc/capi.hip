@@ -257,7 +257,9 @@ size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out
     // one f32[out,in] slice per token chunk of the contraction (one chunk for large layers)
     const size_t slices = mcc::gemm_tn_slices((int)batch, (int)out_features, (int)in_features);
     if (out_features > std::numeric_limits<size_t>::max() / sizeof(float) / in_features / slices) return 0;
-    return slices * out_features * in_features * sizeof(float);
+    // ... and the hand-off words of a contraction that runs as one launch of equal spans
+    return slices * out_features * in_features * sizeof(float) +
+           mcc::gemm_tn_sync_nbytes((int)batch, (int)out_features, (int)in_features);
 }
 
 }  // extern "C"
@@ -361,8 +363,11 @@ int mcc::fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* 
         return fail(MCC_E_INVALID, "compact-counter fused update activation size overflows size_t");
     if (grad_out_nbytes < batch * out_features * sizeof(float) || x_nbytes < batch * in_features * sizeof(float))
         return fail(MCC_E_INVALID, "compact-counter fused update activation buffer is too small");
+    // the hand-off words behind the slices are used when they are there; without them the
+    // contraction is cut up differently and gives the same bits
+    const size_t sync_nbytes = mcc::gemm_tn_sync_nbytes((int)batch, (int)out_features, (int)in_features);
     const size_t full_nbytes = mcc_compact_counter_fused_workspace_nbytes(in_features, out_features, batch);
-    const bool small = workspace_nbytes < full_nbytes;
+    const bool small = workspace_nbytes < full_nbytes - sync_nbytes;
     SmallPlan plan;
     if (small) {
         plan = small_workspace_plan(in_features, out_features, batch);
@@ -415,8 +420,11 @@ int mcc::fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* 
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
         // the chunk slices start at grad_w: the chunk sums are reduced in place into slice 0
+        int* sync_words = sync_nbytes && workspace_nbytes >= full_nbytes
+                              ? reinterpret_cast<int*>(grad_w + out_features * in_features)
+                              : nullptr;
         e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features, grad_w,
-                                    g_contraction_mode.load());
+                                    g_contraction_mode.load(), 0, nullptr, sync_words);
     }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
     {
@@ -512,6 +520,11 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
         jobs[i].k = (int)t.batch;
         jobs[i].m = (int)t.out_features;
         jobs[i].n = (int)t.in_features;
+        // the region ends with the hand-off words of a shape that uses them
+        jobs[i].sync_words = mcc::gemm_tn_sync_nbytes(jobs[i].k, jobs[i].m, jobs[i].n)
+                                 ? reinterpret_cast<int*>(jobs[i].out + mcc::gemm_tn_slices(jobs[i].k, jobs[i].m, jobs[i].n) *
+                                                                           t.out_features * t.in_features)
+                                 : nullptr;
         ws += fused_batched_region(t);
     }
     if (n_tensors > 1) {
@@ -586,13 +599,24 @@ int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, co
         const hipError_t ea = hipMallocAsync(reinterpret_cast<void**>(&temp), slices * m * n * sizeof(float), s);
         if (ea != hipSuccess) return hip_fail(ea, "matmul_transpose_a could not allocate its chunk buffer");
     }
+    int* sync_words = nullptr;
+    const size_t sync_nbytes = mcc::gemm_tn_sync_nbytes((int)k, (int)m, (int)n);
+    if (sync_nbytes && hipMallocAsync(reinterpret_cast<void**>(&sync_words), sync_nbytes, s) != hipSuccess) {
+        (void)hipGetLastError();
+        sync_words = nullptr;  // the contraction runs without them
+    }
     hipError_t e;
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
-        e = mcc::launch_gemm_tn_f32(s, a, b, c, (int)k, (int)m, (int)n, temp, g_contraction_mode.load());
+        e = mcc::launch_gemm_tn_f32(s, a, b, c, (int)k, (int)m, (int)n, temp, g_contraction_mode.load(), 0, nullptr,
+                                    sync_words);
     }
     if (temp) {
         const hipError_t ef = hipFreeAsync(temp, s);
+        if (e == hipSuccess) e = ef;
+    }
+    if (sync_words) {
+        const hipError_t ef = hipFreeAsync(sync_words, s);
         if (e == hipSuccess) e = ef;
     }
     if (e != hipSuccess) return hip_fail(e, "matmul_transpose_a launch failed");

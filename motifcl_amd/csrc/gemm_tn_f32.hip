@@ -217,10 +217,15 @@ GemmTnPlan plan_gemm_tn(int k, int m, int n) {
 
 size_t gemm_tn_slices(int k, int m, int n) { return (size_t)plan_gemm_tn(k, m, n).splits; }
 
+size_t gemm_tn_sync_nbytes(int k, int m, int n) {
+    const GemmTnPlan plan = plan_gemm_tn(k, m, n);
+    return plan.splits == 1 && plan.tile == 128 && gemm_tn_wide_spans_apply(k, m, n) ? kWideSpanWorkgroups * sizeof(int) : 0;
+}
+
 // `slices` holds plan.splits * m * n floats when the plan splits the tokens (it may start at c);
 // it is not touched otherwise.
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c, int k, int m, int n,
-                              float* slices, int mode, int lda, const GemmTnPlan* band_plan) {
+                              float* slices, int mode, int lda, const GemmTnPlan* band_plan, int* sync_words) {
     GemmTnPlan plan = plan_gemm_tn(k, m, n);
     if (band_plan && lda != 0 && lda != m) {
         plan.splits = band_plan->splits;  // the tile size follows the rows at hand (a last, shorter band)
@@ -248,6 +253,8 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
         e = launch_gemm_tn_bf16x6(stream, a, b, out, k, m, n, plan);
     } else if (wide_ok && wide_tiles_fill_the_device(m, n)) {
         e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, n / 256, m / 256, plan.chunk, plan.splits);
+    } else if (wide_ok && plan.splits == 1 && sync_words && gemm_tn_wide_spans_apply(k, m, n)) {
+        e = launch_gemm_tn_wide_spans(stream, a, b, out, k, m, n, sync_words);
     } else if (wide_rows > 0) {
         // wide tiles on the first rows, small tiles on the rest
         const int r = 256 * wide_rows;
@@ -320,7 +327,7 @@ hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_
     for (size_t i = 0; i < n; ++i) {
         if (grouped[i]) continue;
         const hipError_t e = launch_gemm_tn_f32(stream, jobs[i].a, jobs[i].b, jobs[i].out, jobs[i].k, jobs[i].m,
-                                                jobs[i].n, jobs[i].out, 0);
+                                                jobs[i].n, jobs[i].out, 0, 0, nullptr, jobs[i].sync_words);
         if (e != hipSuccess) return e;
     }
     // slices of the grouped tensors, in chunk order

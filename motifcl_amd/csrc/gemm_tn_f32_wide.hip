@@ -1,11 +1,30 @@
 // The weight-gradient contraction c[m,n] = sum_k a[k,m] * b[k,n] on the fp32 matrix cores with
 // 256 x 256 tiles: 8 waves (2 down x 4 across, 128 x 64 each), slabs of 16 tokens copied straight
 // into one of two LDS buffers (global_load_lds_dwordx4).  Against the 128 x 128 tiles of
-// gemm_tn_f32.hip a workgroup copies half as many operand bytes per flop and reads 6 instead of
-// 8 LDS operands per 8 MFMAs.  Every output element still accumulates its tokens in the same
-// order, two at a time, so the result is the same bits.  Whole tiles and whole slabs only.
+// gemm_tn_f32.hip a workgroup copies half as many operand bytes per flop.  Every output element
+// still accumulates its tokens in the same order, two at a time, so the result is the same bits.
+// Whole tiles and whole slabs only.
+//
+// Operand reads.  v_mfma_f32_32x32x2_f32 takes one float per lane from each operand; which matrix
+// row a lane's float belongs to is the kernel's choice.  Here lane l of the wave's four 32-row
+// blocks supplies rows 4 l .. 4 l + 3 (one per block) and columns 2 l, 2 l + 1, so a step's six
+// operand floats are one 16-byte and one 8-byte LDS read instead of six 4-byte ones (+2.7 % on
+// 4096 x 4096 at 32768 tokens: 92 % instead of 90 % of the peak at the measured clock); the
+// accumulators then hold a permuted tile, which the stores undo.  The reads are written as
+// float loads that the compiler merges: a read through a float4 / float2 pointer carries no
+// type-based alias information and makes the compiler wait for the copies of the next slab
+// (s_waitcnt vmcnt(0)) before every first read of a slab, which costs 9 %.
+//
+// Shapes of more than two rounds of tiles that are not whole rounds (11008 x 4096: 688 tiles on
+// 256 CUs) run as one launch of one workgroup per CU in which every workgroup gets the same number
+// of slabs of the (tile, slab) sequence: a partial tile at the end of its span, whole tiles, and a
+// partial tile at the start.  The partial tile at the end is computed first and parked in c; the
+// next workgroup, which owns the rest of that tile, takes it up last, loads the parked
+// accumulators and carries on with the remaining slabs -- the same additions in the same order
+// as an undivided tile, so the same bits, with no last round of idle CUs.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 
 #include "gemm_tile.hpp"
@@ -18,31 +37,38 @@ constexpr int kWide = 256;
 constexpr int kWideThreads = 512;
 constexpr int kWideSlabFloats = kBK * 2 * kWide;  // 16 tokens of both operands: 32 KiB
 
-__global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_kernel(const float* __restrict__ a,
-                                                                       const float* __restrict__ b,
-                                                                       float* __restrict__ c, int K, int M, int N,
-                                                                       int chunk) {
-    __shared__ __attribute__((aligned(1024))) float lds[2 * kWideSlabFloats];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int l32 = lane & 31, half = lane >> 5;
-    const int wm0 = (wave >> 2) * 128, wn0 = (wave & 3) * 64;
-    const TileXY tile = xcd_tile(gridDim.x, gridDim.y, 4);
-    const int m0 = tile.y * kWide, n0 = tile.x * kWide;
-    const int k_begin = blockIdx.z * chunk;
-    const int k_len = K - k_begin < chunk ? K - k_begin : chunk;
-    a += (size_t)k_begin * M + m0;
-    b += (size_t)k_begin * N + n0;
-    c += (size_t)blockIdx.z * M * N;
+struct WideLane {
+    int tid, lane, wave, l32, half, wm0, wn0;
+};
 
-    floatx16 acc[4][2];
+__device__ __forceinline__ WideLane wide_lane() {
+    WideLane t;
+    t.tid = threadIdx.x;
+    t.lane = t.tid & 63;
+    t.wave = t.tid >> 6;
+    t.l32 = t.lane & 31;
+    t.half = t.lane >> 5;
+    t.wm0 = (t.wave >> 2) * 128;
+    t.wn0 = (t.wave & 3) * 64;
+    return t;
+}
+
+typedef floatx16 WideAcc[4][2];
+
+__device__ __forceinline__ void wide_zero(WideAcc& acc) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+}
 
+// acc += the products of k_len tokens (a multiple of 16); a and b point at the first token's row,
+// at the tile's first column.  Ends with every wave past its last LDS read only after the next
+// barrier, so the caller separates two calls by __syncthreads().
+__device__ __forceinline__ void wide_accumulate(const float* __restrict__ a, const float* __restrict__ b, int M, int N,
+                                                int k_len, WideAcc& acc, float* lds, const WideLane& t) {
     typedef __attribute__((address_space(3))) void* lds_ptr;
     typedef const __attribute__((address_space(1))) void* global_ptr;
     // a slab is 32 rows of 1 KiB (16 token rows of a, then 16 of b); wave w copies rows w, w + 8,
@@ -51,14 +77,14 @@ __global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_kernel(const flo
         float* dst = lds + buf * kWideSlabFloats;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int row = wave + 8 * p;
-            __builtin_amdgcn_global_load_lds((global_ptr)(a + (size_t)(k0 + row) * M + 4 * lane),
+            const int row = t.wave + 8 * p;
+            __builtin_amdgcn_global_load_lds((global_ptr)(a + (size_t)(k0 + row) * M + 4 * t.lane),
                                              (lds_ptr)(dst + row * kWide), 16, 0, 0);
         }
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int row = wave + 8 * p;
-            __builtin_amdgcn_global_load_lds((global_ptr)(b + (size_t)(k0 + row) * N + 4 * lane),
+            const int row = t.wave + 8 * p;
+            __builtin_amdgcn_global_load_lds((global_ptr)(b + (size_t)(k0 + row) * N + 4 * t.lane),
                                              (lds_ptr)(dst + (kBK + row) * kWide), 16, 0, 0);
         }
     };
@@ -70,18 +96,16 @@ __global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_kernel(const flo
         if (k0 + kBK < k_len) issue(k0 + kBK, buf ^ 1);
         const float* lds_a = lds + buf * kWideSlabFloats;
         const float* lds_b = lds_a + kBK * kWide;
-        // Operand reads run four steps ahead of the MFMAs that use them: while the next slab is
-        // being copied into LDS a read can take several times its usual latency, and with reads
-        // issued just in time the matrix pipe waits for them (one step ahead: 89.0 % of the peak on
-        // 4096 x 4096, two: 89.8 %, four: 90.3 %, six: 89.9 %).
-        constexpr int D = 4;
+        constexpr int D = 4;  // operand reads run ahead of the MFMAs that use them
         float fa[D + 1][4], fb[D + 1][2];
         auto load = [&](int kk, int set) {
-            const int krow = 2 * kk + half;
+            const int krow = 2 * kk + t.half;
+            const float* pa = &lds_a[krow * kWide + t.wm0 + 4 * t.l32];
+            const float* pb = &lds_b[krow * kWide + t.wn0 + 2 * t.l32];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[set][i] = lds_a[krow * kWide + wm0 + 32 * i + l32];
+            for (int i = 0; i < 4; ++i) fa[set][i] = pa[i];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) fb[set][j] = lds_b[krow * kWide + wn0 + 32 * j + l32];
+            for (int j = 0; j < 2; ++j) fb[set][j] = pb[j];
         };
 #pragma unroll
         for (int q = 0; q < D; ++q) load(q, q);
@@ -93,23 +117,206 @@ __global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_kernel(const flo
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[kk % (D + 1)][i], fb[kk % (D + 1)][j], acc[i][j], 0, 0, 0);
-            if (kk + D < kBK / 2) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+            if (kk + D < kBK / 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
         }
         buf ^= 1;
     }
+}
 
+// acc[i][j][r] is row wm0 + 4 (8 (r/4) + 4 half + r%4) + i, column wn0 + 2 l32 + j of the tile.
+__device__ __forceinline__ void wide_store(float* __restrict__ c, int N, int m0, int n0, const WideAcc& acc,
+                                           const WideLane& t) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = n0 + wn0 + 32 * j + l32;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm0 + 32 * i + 8 * (r / 4) + 4 * half + (r % 4);
-                c[(size_t)row * N + col] = acc[i][j][r];
-            }
+        for (int r = 0; r < 16; ++r) {
+            const int row = m0 + t.wm0 + 4 * (8 * (r / 4) + 4 * t.half + (r % 4)) + i;
+            *reinterpret_cast<float2*>(&c[(size_t)row * N + n0 + t.wn0 + 2 * t.l32]) =
+                make_float2(acc[i][0][r], acc[i][1][r]);
         }
+}
+
+__global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_kernel(const float* __restrict__ a,
+                                                                       const float* __restrict__ b,
+                                                                       float* __restrict__ c, int K, int M, int N,
+                                                                       int chunk) {
+    __shared__ __attribute__((aligned(1024))) float lds[2 * kWideSlabFloats];
+    const WideLane t = wide_lane();
+    const TileXY tile = xcd_tile(gridDim.x, gridDim.y, 4);
+    const int m0 = tile.y * kWide, n0 = tile.x * kWide;
+    const int k_begin = blockIdx.z * chunk;
+    const int k_len = K - k_begin < chunk ? K - k_begin : chunk;
+    WideAcc acc;
+    wide_zero(acc);
+    wide_accumulate(a + (size_t)k_begin * M + m0, b + (size_t)k_begin * N + n0, M, N, k_len, acc, lds, t);
+    wide_store(c + (size_t)blockIdx.z * M * N, N, m0, n0, acc, t);
+}
+
+// ---------------------------------------------------------------------------- equal spans
+// Hand-off word of workgroup j's parked tile: 0 nothing yet, kWriting the owner is storing it,
+// kParked it is complete, kAbandoned the taker has given up waiting and computes the whole tile
+// itself (the owner then skips its stores).  Every transition is a compare-and-swap from 0, so
+// exactly one side wins; the parked accumulators cross the per-XCD L2 caches as device-scope atomic
+// accesses, ordered by completion (the owner's stores are acknowledged before it raises the word,
+// the taker loads after it has seen it).
+constexpr int kWriting = 3, kParked = 1, kAbandoned = 2;
+
+__device__ __forceinline__ int word_load(const int* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool word_claim(int* p, int desired) {
+    int expected = 0;
+    return __hip_atomic_compare_exchange_strong(p, &expected, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The 65536 accumulators of a tile in the order (register, thread): element q * 512 + tid of the
+// tile read row by row, so a wave moves whole 256-byte pieces.
+__device__ __forceinline__ void wide_park(float* __restrict__ c, int N, int m0, int n0, const WideAcc& acc, int tid) {
+#pragma unroll
+    for (int q = 0; q < 128; ++q) {
+        const int idx = q * kWideThreads + tid;
+        __hip_atomic_store(&c[(size_t)(m0 + (idx >> 8)) * N + n0 + (idx & 255)], acc[q / 32][(q / 16) % 2][q % 16],
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+__device__ __forceinline__ void wide_take(const float* __restrict__ c, int N, int m0, int n0, WideAcc& acc, int tid) {
+#pragma unroll
+    for (int q = 0; q < 128; ++q) {
+        const int idx = q * kWideThreads + tid;
+        acc[q / 32][(q / 16) % 2][q % 16] = __hip_atomic_load(&c[(size_t)(m0 + (idx >> 8)) * N + n0 + (idx & 255)],
+                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// Tiles in bands of four tile rows, column by column inside a band, so that workgroups with
+// neighbouring spans work on tiles that share operand panels.
+__device__ __forceinline__ TileXY band_tile(int t, int tiles_x, int tiles_y) {
+    const int band_tiles = 4 * tiles_x;
+    const int band = t / band_tiles, within = t - band * band_tiles;
+    const int left = tiles_y - 4 * band;
+    const int rows = left < 4 ? left : 4;
+    TileXY r;
+    r.x = within / rows;
+    r.y = 4 * band + within % rows;
+    return r;
+}
+
+__global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_spans_kernel(
+    const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ c, int K, int M, int N, int tiles_x,
+    int tiles_y, int* words, unsigned spin_limit, int start_first) {
+    // One LDS object, read and written as floats only: a second LDS variable gives every LDS access
+    // alias-scope metadata, and an access of another type loses the type-based one; with either
+    // the compiler waits for the slab copies in flight (s_waitcnt vmcnt(0)) before the operand
+    // reads of the slab at hand, which serialises copy and arithmetic.
+    __shared__ __attribute__((aligned(1024))) float lds[2 * kWideSlabFloats + 64];
+    float& verdict = lds[2 * kWideSlabFloats];
+    const WideLane t = wide_lane();
+    // workgroups w, w + 8, ... share an XCD (and its L2): give them neighbouring spans
+    const int P = gridDim.x;
+    const int j = (P & 7) == 0 ? (int)(blockIdx.x & 7u) * (P >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const long spt = K / kBK;  // slabs per tile
+    const long total = (long)tiles_x * tiles_y * spt;
+    const long base = total / P, rem = total % P;
+    const long begin = j * base + (j < rem ? j : rem);
+    const long end = begin + base + (j < rem ? 1 : 0);
+    const int first_tile = (int)(begin / spt), last_tile = (int)((end - 1) / spt);
+    const int s0 = (int)(begin - first_tile * spt);     // slabs of first_tile that belong to the span before
+    const int e1 = (int)(end - (long)last_tile * spt);  // slabs of last_tile inside this span
+    const bool has_start = s0 > 0, has_end = e1 < spt;  // the span is longer than two tiles: never the same tile
+    WideAcc acc;
+
+    auto tile_origin = [&](int tile, int& m0, int& n0) {
+        const TileXY xy = band_tile(tile, tiles_x, tiles_y);
+        m0 = xy.y * kWide;
+        n0 = xy.x * kWide;
+    };
+    // the partial tile at the end of the span: slabs [0, e1), parked in c for workgroup j + 1
+    auto run_end = [&]() {
+        int m0, n0;
+        tile_origin(last_tile, m0, n0);
+        wide_zero(acc);
+        __syncthreads();
+        wide_accumulate(a + m0, b + n0, M, N, e1 * kBK, acc, lds, t);
+        if (t.tid == 0) verdict = word_claim(&words[j], kWriting) ? 1.0f : 0.0f;
+        __syncthreads();
+        if (verdict != 0.0f) {  // else the taker has given up and computes the tile alone
+            wide_park(c, N, m0, n0, acc, t.tid);
+            __builtin_amdgcn_s_waitcnt(0);  // stores acknowledged
+            __syncthreads();
+            if (t.tid == 0) __hip_atomic_store(&words[j], kParked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+    };
+    auto run_whole = [&]() {
+        for (int tile = first_tile + (has_start ? 1 : 0); tile <= last_tile - (has_end ? 1 : 0); ++tile) {
+            int m0, n0;
+            tile_origin(tile, m0, n0);
+            wide_zero(acc);
+            __syncthreads();
+            wide_accumulate(a + m0, b + n0, M, N, K, acc, lds, t);
+            wide_store(c, N, m0, n0, acc, t);
+        }
+    };
+    // the partial tile at the start: slabs [s0, spt) on top of what workgroup j - 1 parked
+    auto run_start = [&]() {
+        int m0, n0;
+        tile_origin(first_tile, m0, n0);
+        if (t.tid == 0) {
+            int* word = &words[j - 1];
+            int got = 0;
+            unsigned polls = 0;
+            for (;;) {
+                const int seen = word_load(word);
+                if (seen == kParked) { got = 1; break; }
+                // kWriting: the owner is running and about to finish, whatever the budget says
+                if (seen == 0 && polls >= spin_limit && word_claim(word, kAbandoned)) break;
+                __builtin_amdgcn_s_sleep(32);
+                ++polls;
+            }
+            verdict = got ? 1.0f : 0.0f;
+        }
+        __syncthreads();
+        const bool parked = verdict != 0.0f;
+        if (parked) wide_take(c, N, m0, n0, acc, t.tid); else wide_zero(acc);
+        const int from = parked ? s0 : 0;
+        __syncthreads();
+        wide_accumulate(a + (size_t)from * kBK * M + m0, b + (size_t)from * kBK * N + n0, M, N, (int)(spt - from) * kBK,
+                        acc, lds, t);
+        wide_store(c, N, m0, n0, acc, t);
+    };
+    if (!start_first) {
+        if (has_end) run_end();
+        run_whole();
+        if (has_start) run_start();
+    } else {  // test order: every taker arrives before its owner
+        if (has_start) run_start();
+        run_whole();
+        if (has_end) run_end();
+    }
+}
+
+__global__ void clear_words_kernel(int* words, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) words[i] = 0;
+}
+
+// about 0.9 us per poll: 4 ms before a taker computes a tile alone
+constexpr unsigned kDefaultSpanPolls = 4096;
+std::atomic<unsigned> g_span_polls{kDefaultSpanPolls};
+std::atomic<int> g_span_start_first{0};
+
+int device_cus() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    int cus = cached[dev].load();
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev].store(cus);
+    }
+    return cus;
 }
 
 }  // namespace
@@ -125,6 +332,30 @@ hipError_t launch_gemm_tn_wide(hipStream_t stream, const float* a, const float* 
     const dim3 grid(tiles_x, tiles_y, splits);
     hipLaunchKernelGGL(gemm_tn_wide_kernel, grid, dim3(kWideThreads), 0, stream, a, b, out, k, m, n, chunk);
     return hipGetLastError();
+}
+
+bool gemm_tn_wide_spans_apply(int k, int m, int n) {
+    if (m % kWide || n % kWide || k % kBK) return false;
+    const long tiles = (long)(m / kWide) * (n / kWide);
+    return tiles > 2 * kWideSpanWorkgroups && tiles % kWideSpanWorkgroups != 0;
+}
+
+hipError_t launch_gemm_tn_wide_spans(hipStream_t stream, const float* a, const float* b, float* out, int k, int m,
+                                     int n, int* words) {
+    // one workgroup per CU; on a device of another size the spans are simply longer or shorter
+    int wgs = device_cus();
+    if (wgs <= 0 || wgs > kWideSpanWorkgroups) wgs = kWideSpanWorkgroups;
+    const long tiles = (long)(m / kWide) * (n / kWide);
+    if (tiles < 2L * wgs) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(kWideSpanWorkgroups), 0, stream, words, kWideSpanWorkgroups);
+    hipLaunchKernelGGL(gemm_tn_wide_spans_kernel, dim3(wgs), dim3(kWideThreads), 0, stream, a, b, out, k, m, n,
+                       n / kWide, m / kWide, words, g_span_polls.load(), g_span_start_first.load());
+    return hipGetLastError();
+}
+
+void set_gemm_tn_wide_spans_test_mode(unsigned polls, int start_first) {
+    g_span_polls.store(polls == 0xffffffffu ? kDefaultSpanPolls : polls);
+    g_span_start_first.store(start_first ? 1 : 0);
 }
 
 }  // namespace mcc

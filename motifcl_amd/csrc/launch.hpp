@@ -54,17 +54,32 @@ struct GemmTnPlan {
 };
 GemmTnPlan plan_gemm_tn(int k, int m, int n);
 size_t gemm_tn_slices(int k, int m, int n);
+// Bytes of hand-off words a contraction of this shape can use beyond its slices (0: none): shapes
+// of more than two rounds of 256 x 256 tiles that are not whole rounds run as one launch of equal
+// spans (gemm_tn_f32_wide.hip) when the caller lends them.
+size_t gemm_tn_sync_nbytes(int k, int m, int n);
 // mode: 0 = fp32 matrix instruction; 1 = both operands split into three bf16 terms, six bf16
 // passes (gemm_tn_bf16x6.hip), where the shape allows it
 // lda: floats between rows of a (0 = m); a wider lda contracts a column band of a [k, lda] matrix,
 // cut up as `band_plan` says (the caller sized `slices` for it) instead of by the band's own shape
+// sync_words: gemm_tn_sync_nbytes bytes of device memory, or null (the result is the same bits)
 hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b, float* c,
                               int k, int m, int n, float* slices, int mode = 0, int lda = 0,
-                              const GemmTnPlan* band_plan = nullptr);
+                              const GemmTnPlan* band_plan = nullptr, int* sync_words = nullptr);
 // 256 x 256-tile form of the contraction for whole tiles (gemm_tn_f32_wide.hip)
 bool gemm_tn_wide_supports(const float* a, const float* b, int k, int m, int n, int chunk);
 hipError_t launch_gemm_tn_wide(hipStream_t stream, const float* a, const float* b, float* out, int k, int m, int n,
                                int tiles_x, int tiles_y, int chunk, int splits);
+// The whole contraction as one launch of at most kWideSpanWorkgroups workgroups with equal spans of
+// the (tile, slab) sequence; `words` holds kWideSpanWorkgroups ints (cleared by the launch).
+constexpr int kWideSpanWorkgroups = 256;
+bool gemm_tn_wide_spans_apply(int k, int m, int n);
+hipError_t launch_gemm_tn_wide_spans(hipStream_t stream, const float* a, const float* b, float* out, int k, int m,
+                                     int n, int* words);
+// Test aid (motifcl_amd_diag.h): polls a workgroup spends on a parked tile before it computes the
+// tile alone (0xffffffff restores the default), and whether workgroups take up the tile begun by
+// their neighbour before instead of after their own tiles, so that every wait runs out.
+void set_gemm_tn_wide_spans_test_mode(unsigned polls, int start_first);
 
 // One contraction of a grouped launch: out holds gemm_tn_slices(k, m, n) matrices of m*n floats,
 // the result ends up in the first.
@@ -73,6 +88,7 @@ struct GemmTnJob {
     const float* b;  // [k, n]
     float* out;
     int k, m, n;
+    int* sync_words = nullptr;  // as for launch_gemm_tn_f32
 };
 hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_t n);
 
