@@ -205,7 +205,7 @@ __device__ __forceinline__ TileXY band_tile(int t, int tiles_x, int tiles_y) {
 
 __global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_spans_kernel(
     const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ c, int K, int M, int N, int tiles_x,
-    int tiles_y, int* words, unsigned spin_limit, int start_first) {
+    int tiles_y, int* words, unsigned spin_limit, int start_first, int classes, int order) {
     // One LDS object, read and written as floats only: a second LDS variable gives every LDS access
     // alias-scope metadata, and an access of another type loses the type-based one; with either
     // the compiler waits for the slab copies in flight (s_waitcnt vmcnt(0)) before the operand
@@ -213,9 +213,20 @@ __global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_spans_kernel(
     __shared__ __attribute__((aligned(1024))) float lds[2 * kWideSlabFloats + 64];
     float& verdict = lds[2 * kWideSlabFloats];
     const WideLane t = wide_lane();
-    // workgroups w, w + 8, ... share an XCD (and its L2): give them neighbouring spans
+    // Workgroups w, w + 8, ... share an XCD and its L2, which holds a few slabs of the panels in
+    // use: two workgroups share a panel's fetches only while they are at the same token.  Spans
+    // j, j + classes, j + 2 classes, ... begin whole tiles at the same moment (their first pieces
+    // are equally long), so an XCD gets all spans of classes / 8 such families and the tile order
+    // puts their tiles on one line of the tile grid (classes == 0: no such structure, neighbouring
+    // spans per XCD).
     const int P = gridDim.x;
-    const int j = (P & 7) == 0 ? (int)(blockIdx.x & 7u) * (P >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    int j = (int)blockIdx.x;
+    if (classes > 0) {
+        const int per_xcd = classes >> 3, local = (int)(blockIdx.x >> 3);
+        j = (local / per_xcd) * classes + (int)(blockIdx.x & 7u) * per_xcd + local % per_xcd;
+    } else if ((P & 7) == 0) {
+        j = (int)(blockIdx.x & 7u) * (P >> 3) + (int)(blockIdx.x >> 3);
+    }
     const long spt = K / kBK;  // slabs per tile
     const long total = (long)tiles_x * tiles_y * spt;
     const long base = total / P, rem = total % P;
@@ -228,7 +239,10 @@ __global__ __launch_bounds__(kWideThreads, 2) void gemm_tn_wide_spans_kernel(
     WideAcc acc;
 
     auto tile_origin = [&](int tile, int& m0, int& n0) {
-        const TileXY xy = band_tile(tile, tiles_x, tiles_y);
+        TileXY xy;
+        if (order == 1) { xy.y = tile % tiles_y; xy.x = tile / tiles_y; }
+        else if (order == 2) { xy.x = tile % tiles_x; xy.y = tile / tiles_x; }
+        else xy = band_tile(tile, tiles_x, tiles_y);
         m0 = xy.y * kWide;
         n0 = xy.x * kWide;
     };
@@ -306,6 +320,7 @@ __global__ void clear_words_kernel(int* words, int n) {
 constexpr unsigned kDefaultSpanPolls = 4096;
 std::atomic<unsigned> g_span_polls{kDefaultSpanPolls};
 std::atomic<int> g_span_start_first{0};
+std::atomic<int> g_span_order_override{-1};
 
 int device_cus() {
     static std::atomic<int> cached[64];
@@ -348,14 +363,31 @@ hipError_t launch_gemm_tn_wide_spans(hipStream_t stream, const float* a, const f
     const long tiles = (long)(m / kWide) * (n / kWide);
     if (tiles < 2L * wgs) return hipErrorInvalidValue;
     hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(kWideSpanWorkgroups), 0, stream, words, kWideSpanWorkgroups);
+    // spans j and j + g start at the same slab of their tiles when g spans are a whole number of
+    // tiles; with the tiles of such a family one line of the grid apart they share a panel
+    const int tiles_x = n / kWide, tiles_y = m / kWide;
+    const long spt = k / kBK, total = tiles * spt;
+    int classes = 0, order = 0;
+    if (total % wgs == 0 && wgs % 8 == 0) {
+        const long base = total / wgs;
+        long g = 1;
+        while (g <= wgs && (base * g) % spt) ++g;
+        const long step = base * g / spt;  // tiles between spans of a family
+        if (g <= wgs && g % 8 == 0 && wgs % g == 0 && (step == tiles_y || step == tiles_x)) {
+            classes = (int)g;
+            order = step == tiles_y ? 1 : 2;
+        }
+    }
+    if (g_span_order_override.load() >= 0) { classes = 0; order = 0; }
     hipLaunchKernelGGL(gemm_tn_wide_spans_kernel, dim3(wgs), dim3(kWideThreads), 0, stream, a, b, out, k, m, n,
-                       n / kWide, m / kWide, words, g_span_polls.load(), g_span_start_first.load());
+                       tiles_x, tiles_y, words, g_span_polls.load(), g_span_start_first.load(), classes, order);
     return hipGetLastError();
 }
 
 void set_gemm_tn_wide_spans_test_mode(unsigned polls, int start_first) {
     g_span_polls.store(polls == 0xffffffffu ? kDefaultSpanPolls : polls);
-    g_span_start_first.store(start_first ? 1 : 0);
+    g_span_start_first.store(start_first & 1);
+    g_span_order_override.store((start_first & 2) ? 0 : -1);
 }
 
 }  // namespace mcc
