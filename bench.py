@@ -14,7 +14,7 @@ fused update of all seven tensors.  The same JSON line carries
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg0|cfg1|cfg2|cfg4]
                     [--fused-path workspace|strip] [--batched] [--graph]
-                    [--no-update-only] [--no-small] [--no-cpu] [--no-clock]
+                    [--no-update-only] [--no-small] [--no-by-row-length] [--no-cpu] [--no-clock]
 
 Inputs are synthetic, from the library's counter-based generator (lowbias32 of element index
 and stream id -> Box-Muller; mcc_fill_normal_f32 / mcc_fill_counter_state_u8), seed 0:
@@ -43,13 +43,14 @@ C, LR, LR_SCALE, BETA, EPS = 11, 3e-3, 0.0, 0.9, 1e-3
 BYTES_PER_PARAM = 5.5          # 4 (read G) + 0.75 (read state) + 0.75 (write state)
 SEED = 0
 
-# HBM-side bytes per launch of the dominant kernels, from `rocprofv3 --pmc FETCH_SIZE` /
-# `--pmc WRITE_SIZE` runs of this same command (scaled by a plain 1 GiB copy).  They are reported
-# with their source, not re-measured in the run.
+# HBM-side bytes per launch of the dominant kernels (for the fused step: the step's bytes over its
+# seven contraction launches), from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this
+# same command (scaled by a plain 1 GiB copy).  They are reported with their source, not
+# re-measured in the run.
 MEASURED_TRAFFIC = {
-    "cfg4/gemm_tn_f32": (8.94e9, "profiles/gemm_tn_f32__cfg4_fused_step.txt"),
-    "cfg4/fused_strip": (27.53e9, "profiles/fused_strip__cfg4_fused_step.txt"),
-    "cfg3/update_rows": (36.16e9, "profiles/update_rows__cfg3_update_only.txt"),
+    "cfg4/gemm_tn_f32": (1.140e10, "profiles/gemm_tn_f32__cfg4_fused_step.txt"),
+    "cfg4/fused_strip": (3.204e10, "profiles/fused_strip__cfg4_fused_step.txt"),
+    "cfg3/update_rows": (3.650e10, "profiles/update_rows__cfg3_update_only.txt"),
 }
 
 
@@ -373,7 +374,7 @@ def bench_side_optimizer(L, ops, steps, warmup):
 
 
 # ------------------------------------------------------------------------------ update-only step
-def bench_update_only(L, ops, steps, warmup):
+def bench_update_only(L, ops, steps, warmup, by_row_length=True):
     import torch
     shapes = layer_shapes(4096, 11008)
     layers = 32
@@ -420,7 +421,7 @@ def bench_update_only(L, ops, steps, warmup):
     }
     # by row length: the 4096-wide rows (one wave per row) and the 11008-wide rows (four waves per row)
     by_width = {}
-    for width in (4096, 11008):
+    for width in ((4096, 11008) if by_row_length else ()):
         sub = [(st[0], st[1], st[2], g) for (st, g, _, n_in) in tensors if n_in == width][:32]
         sub_params = sum(t[3].numel() for t in sub)
         sb = ops.UpdateBatch(sub, LR, list(range(len(sub))))
@@ -636,6 +637,8 @@ def main():
                     help="fused leg through mcc_compact_counter_apply_update_fused_batched (one call per step)")
     ap.add_argument("--no-update-only", action="store_true", help="skip the cfg3 update-only leg")
     ap.add_argument("--no-small", action="store_true", help="skip the cfg0-cfg2 legs")
+    ap.add_argument("--no-by-row-length", action="store_true",
+                    help="skip the update-only sub-legs by row length (counter runs want the cfg3 launches only)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the legs beside the path (split-bf16 contraction, layer products, side optimizer)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs and the parity checks that need them")
@@ -723,7 +726,7 @@ def main():
         line["layer_products"] = bench_layer_products(L, ops, args.workload, max(2, args.steps // 2), 1)
         torch.cuda.empty_cache()
     if not args.no_update_only:
-        uo, uo_tensors = bench_update_only(L, ops, args.steps, args.warmup)
+        uo, uo_tensors = bench_update_only(L, ops, args.steps, args.warmup, not args.no_by_row_length)
         if not args.no_cpu:
             uo["cpu_baseline"] = cpu_baseline_dense(uo_tensors[0])
             uo["parity_full_size"] = parity_full_size_update_only(ops, uo_tensors)
