@@ -1,0 +1,64 @@
+"""The two 7B-shaped BASELINE configs at their real sizes, against the CPU oracle.
+
+cfg4: one [4096, 4096] tensor of the layer at the full 32768 tokens -- the contraction within
+1e-4 of the oracle's sequential fp32 sum, state / scale / v bit-exact given the GPU's own gradient,
+and the fraction of counters that land on another code than the oracle's reported and bounded.
+cfg3: one tensor of each shape of the 224 at full size, update-only, bit-exact.
+The oracle needs a few seconds per case on 16 threads."""
+import numpy as np
+import pytest
+import torch
+
+from tests.test_gpu_parity import ops  # noqa: F401  (fixture)
+
+pytestmark = pytest.mark.gpu
+C, LR, BETA, EPS = 11, 3e-3, 0.9, 1e-3
+
+
+def make_state(ops, n_out, n_in, stream):
+    state = ops.fill_counter_state(torch.empty(n_out * n_in // 4 * 3, dtype=torch.uint8, device="cuda"), stream, 63)
+    scale = torch.full((n_out,), float(np.sqrt(3.0 / (2.0 * n_in))), dtype=torch.float32, device="cuda")
+    v = torch.zeros(n_out, dtype=torch.float32, device="cuda")
+    return state, scale, v
+
+
+@pytest.mark.parametrize("lr_scale", [0.0, 0.05])
+def test_cfg4_tensor_at_32768_tokens_against_the_oracle(ops, oracle, lr_scale):
+    tokens, n_out, n_in = 32768, 4096, 4096
+    x = ops.fill_normal(torch.empty(tokens, n_in, device="cuda"), 101, 1.0)
+    dy = ops.fill_normal(torch.empty(tokens, n_out, device="cuda"), 102, 0.01)
+    st = make_state(ops, n_out, n_in, 103)
+    h0 = [t.cpu().numpy().copy() for t in st]
+    ws = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, tokens), dtype=torch.uint8, device="cuda")
+    ops.apply_update_fused(st[0], st[1], st[2], dy, x, ws, C, LR, lr_scale, BETA, EPS, 4242)
+    torch.cuda.synchronize()
+    got = [t.cpu().numpy() for t in st]
+    g_gpu = ws.view(torch.float32)[: n_out * n_in].view(n_out, n_in).cpu().numpy()
+    e_state, e_scale, e_v, g_seq = oracle.update_fused(h0[0], h0[1], h0[2], dy.cpu().numpy(), x.cpu().numpy(), C, LR,
+                                                      lr_scale, BETA, EPS, 4242)
+    rel = np.abs(g_gpu - g_seq).max() / np.abs(g_seq).max()
+    assert rel <= 1e-4, rel
+    x_state, x_scale, x_v = oracle.update_dense(h0[0], h0[1], h0[2], g_gpu, C, LR, lr_scale, BETA, EPS, 4242)
+    assert np.array_equal(got[0], x_state) and np.array_equal(got[1], x_scale) and np.array_equal(got[2], x_v)
+    flips = float((oracle.unpack_codes(got[0]) != oracle.unpack_codes(e_state)).mean())
+    print("cfg4 [4096,4096]@32768 lr_scale=%g: max|dG|/max|G| = %.2e, flip fraction = %.2e" % (lr_scale, rel, flips))
+    assert flips <= 1e-4
+    # scale moves by lr_scale * (sum of g t) / sqrt(in), a sum with cancellation: compare on the scale's own size
+    print("    scale: max abs diff %.2e of max %.2e; v: max rel diff %.2e" % (
+        np.abs(got[1] - e_scale).max(), np.abs(e_scale).max(), (np.abs(got[2] - e_v) / e_v).max()))
+    assert np.abs(got[1] - e_scale).max() <= 1e-5 * np.abs(e_scale).max()
+    np.testing.assert_allclose(got[2], e_v, rtol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (11008, 4096), (4096, 11008)], ids=lambda s: "%dx%d" % s)
+def test_cfg3_tensor_update_only_is_bit_exact(ops, oracle, shape):
+    n_out, n_in = shape
+    g = ops.fill_normal(torch.empty(n_out, n_in, device="cuda"), 201, 0.01)
+    st = make_state(ops, n_out, n_in, 202)
+    h0 = [t.cpu().numpy().copy() for t in st]
+    ops.apply_update_dense(st[0], st[1], st[2], g, C, LR, 0.0, BETA, EPS, 777)
+    torch.cuda.synchronize()
+    exp = oracle.update_dense(h0[0], h0[1], h0[2], g.cpu().numpy(), C, LR, 0.0, BETA, EPS, 777)
+    for a, b in zip([t.cpu().numpy() for t in st], exp):
+        assert np.array_equal(a, b)
+    assert float((oracle.unpack_codes(exp[0]) != oracle.unpack_codes(h0[0])).mean()) > 0.5  # the step did something
