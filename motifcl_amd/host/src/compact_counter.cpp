@@ -19,33 +19,54 @@
 namespace motifcl::nn {
 namespace {
 
-inline std::uint8_t cc_encode(int t, int c, int C) {
-    const int lv = 2 * C - 1;
-    return static_cast<std::uint8_t>((t + 1) * lv + (c + (C - 1)));
+// Packed start state: every weight a ternary value drawn from {-1, 0, +1} with its counter at
+// zero, code = (t + 1)(2C - 1) + (C - 1), four codes to a little-endian 24-bit word.  The draws
+// are MotifCL's (std::mt19937(seed) through uniform_int_distribution<int>(-1, 1), row-major), so
+// a layer built with the same seed and standard library starts from the same weights.
+std::vector<std::uint8_t> initial_state(int out_features, int in_features, int C, std::uint32_t seed) {
+    const std::size_t groups = static_cast<std::size_t>(out_features) * (in_features / 4);
+    const std::uint32_t zero_counter = static_cast<std::uint32_t>(C - 1), levels = static_cast<std::uint32_t>(2 * C - 1);
+    std::mt19937 rng(seed);
+    std::uniform_int_distribution<int> ternary(-1, 1);
+    std::vector<std::uint8_t> bytes(groups * 3);
+    for (std::size_t g = 0; g < groups; ++g) {
+        std::uint32_t word = 0;
+        for (int k = 0; k < 4; ++k)
+            word |= (static_cast<std::uint32_t>(ternary(rng) + 1) * levels + zero_counter) << (6 * k);
+        bytes[3 * g] = static_cast<std::uint8_t>(word);
+        bytes[3 * g + 1] = static_cast<std::uint8_t>(word >> 8);
+        bytes[3 * g + 2] = static_cast<std::uint8_t>(word >> 16);
+    }
+    return bytes;
 }
 
+// What backward does for a counter layer (src/nn/compact_counter.cpp:30-51): the input gradient is
+// taken from the state the forward pass saw, then the state is updated -- immediately, or recorded
+// for one batched call -- and only then does the input's own backward run.  The update happens
+// whether or not the input wants a gradient, so a layer fed with raw data still learns.
 struct CounterBackwardNode : autograd::Node {
-    Tensor x;
-    CounterStateLinear* layer;
-    std::uint32_t seed;
+    CounterBackwardNode(Tensor input, CounterStateLinear* owner, std::uint32_t update_seed)
+        : input_(std::move(input)), owner_(owner), update_seed_(update_seed) {}
 
-    CounterBackwardNode(Tensor x_, CounterStateLinear* l, std::uint32_t s) : x(std::move(x_)), layer(l), seed(s) {}
-
-    std::vector<Tensor> inputs() const override { return {x}; }
+    std::vector<Tensor> inputs() const override { return {input_}; }
 
     void backward(const Tensor& grad_out) override {
-        const bool need_gx = x.requires_grad();
-        Tensor grad_x;
-        if (need_gx) grad_x = layer->backward_input_from_state(grad_out);  // PRE-update state
+        Tensor grad_input;
+        if (input_.requires_grad()) grad_input = owner_->backward_input_from_state(grad_out);
         {
-            autograd::NoGradGuard guard;
-            if (layer->deferred())
-                layer->deferred()->add(*layer, grad_out, x, seed);
+            autograd::NoGradGuard no_graph;  // the update is a side effect, not part of the graph
+            if (DeferredCounterUpdates* pending = owner_->deferred())
+                pending->add(*owner_, grad_out, input_, update_seed_);
             else
-                layer->apply_update_backward(grad_out, x, seed);
+                owner_->apply_update_backward(grad_out, input_, update_seed_);
         }
-        if (need_gx) x.backward(grad_x);
+        if (grad_input.valid()) input_.backward(grad_input);
     }
+
+private:
+    Tensor input_;
+    CounterStateLinear* owner_;
+    std::uint32_t update_seed_;
 };
 
 const float* f32(const Tensor& t) { return static_cast<const float*>(t.data()); }
@@ -58,30 +79,19 @@ CounterStateLinear::CounterStateLinear(Backend& backend, int in_features, int ou
                                        std::uint32_t seed)
     : backend_(&backend), in_(in_features), out_(out_features), C_(C), lr_(lr), lr_scale_(lr_scale),
       rms_beta_(rms_beta), rms_eps_(rms_eps), seed_(seed) {
+    // the reference's conditions and messages (src/nn/compact_counter.cpp:60-62)
     MCL_CHECK(in_ > 0 && out_ > 0, "CounterStateLinear requires positive dimensions");
     MCL_CHECK(C_ > 0 && 3 * (2 * C_ - 1) <= 64, "C too large for 6-bit packed state encoding");
     MCL_CHECK(in_ % 4 == 0, "CounterStateLinear requires in_features divisible by 4 (6-bit packing)");
 
-    std::mt19937 rng(seed);
-    std::uniform_int_distribution<int> tern(-1, 1);
-    const int gpr = in_ / 4;
-    std::vector<std::uint8_t> st(static_cast<std::size_t>(out_) * gpr * 3);
-    for (int row = 0; row < out_; ++row)
-        for (int g = 0; g < gpr; ++g) {
-            std::uint32_t word = 0;
-            for (int k = 0; k < 4; ++k) word |= static_cast<std::uint32_t>(cc_encode(tern(rng), 0, C_)) << (6 * k);
-            std::uint8_t* p = st.data() + (static_cast<std::size_t>(row) * gpr + g) * 3;
-            p[0] = static_cast<std::uint8_t>(word & 0xFF);
-            p[1] = static_cast<std::uint8_t>((word >> 8) & 0xFF);
-            p[2] = static_cast<std::uint8_t>((word >> 16) & 0xFF);
-        }
-    state = Tensor::from_cpu(*backend_, {static_cast<int64_t>(out_) * gpr * 3}, DType::U8, st.data());
-
-    const float s0 = init_gain * std::sqrt(3.0f / (2.0f * static_cast<float>(in_)));
-    std::vector<float> sc(static_cast<std::size_t>(out_), s0);
-    std::vector<float> vv(static_cast<std::size_t>(out_), 0.0f);
-    scale = Tensor::from_cpu(*backend_, {out_}, DType::F32, sc.data());
-    v = Tensor::from_cpu(*backend_, {out_}, DType::F32, vv.data());
+    const std::vector<std::uint8_t> packed = initial_state(out_, in_, C_, seed);
+    state = Tensor::from_cpu(*backend_, {static_cast<int64_t>(packed.size())}, DType::U8, packed.data());
+    // every row starts at init_gain * sqrt(3 / (2 in)) with an empty second moment
+    const std::vector<float> start_scale(static_cast<std::size_t>(out_),
+                                         init_gain * std::sqrt(3.0f / (2.0f * static_cast<float>(in_))));
+    const std::vector<float> zeros(static_cast<std::size_t>(out_), 0.0f);
+    scale = Tensor::from_cpu(*backend_, {out_}, DType::F32, start_scale.data());
+    v = Tensor::from_cpu(*backend_, {out_}, DType::F32, zeros.data());
 }
 
 Tensor CounterStateLinear::decode_weight() const {

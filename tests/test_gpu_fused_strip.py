@@ -159,12 +159,14 @@ def test_small_workspace_rules(ops):
 def test_second_strip_step_on_another_stream_is_refused_while_the_first_runs(ops):
     # tiles of a strip wait for each other on the device, so two such launches must not share the GPU
     from motifcl_amd.lib import MccError
-    n, n_in, n_out, C = 8192, 4096, 4096, 11
+    n, n_in, n_out, C = 16384, 4096, 4096, 11
     rng = np.random.default_rng(0)
     state = dev(rng.integers(0, 63, n_out * n_in // 4 * 3).astype(np.uint8))
-    state2 = state.clone()
     scale = torch.full((n_out,), 0.02, device="cuda")
     v = torch.zeros(n_out, device="cuda")
+    # everything the second call touches exists before the first is launched: an allocation in
+    # between may wait for the device, and the first step would be over before the second is tried
+    state2, scale2, v2 = state.clone(), scale.clone(), v.clone()
     x = torch.randn(n, n_in, device="cuda")
     dy = torch.randn(n, n_out, device="cuda") * 0.01
     nbytes = ops.fused_strip_workspace_nbytes(n_in, n_out, n)
@@ -172,17 +174,18 @@ def test_second_strip_step_on_another_stream_is_refused_while_the_first_runs(ops
     ws2 = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     side = torch.cuda.Stream()
     torch.cuda.synchronize()
-    ops.apply_update_fused(state, scale, v, dy, x, ws1, C, 3e-3, 0.0, 0.9, 1e-3, 1)  # about 1.5 ms of work
+    ops.apply_update_fused(state, scale, v, dy, x, ws1, C, 3e-3, 0.0, 0.9, 1e-3, 1)  # about 4.5 ms of work
     with torch.cuda.stream(side):
         with pytest.raises(MccError, match="different stream"):
-            ops.apply_update_fused(state2, scale.clone(), v.clone(), dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
+            ops.apply_update_fused(state2, scale2, v2, dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
     torch.cuda.synchronize()
     ops.fused_check(ws1, n_in, n_out, n)
     # once the first has finished the other stream may go
     with torch.cuda.stream(side):
-        ops.apply_update_fused(state2, scale.clone(), v.clone(), dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
+        ops.apply_update_fused(state2, scale2, v2, dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
     torch.cuda.synchronize()
     ops.fused_check(ws2, n_in, n_out, n)
+    assert torch.equal(state, state2) and torch.equal(scale, scale2) and torch.equal(v, v2)
 
 
 def test_two_strip_updates_in_a_row_are_deterministic(ops):
