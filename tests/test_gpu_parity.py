@@ -144,10 +144,13 @@ def test_update_dense_batched_matches_per_tensor_oracle(ops, oracle):
         assert_bit_exact([host(t) for t in dev_tensors[i][:3]], exp)
 
 
-def test_tiny_and_huge_gradients_take_the_exact_division(ops, oracle):
+@pytest.mark.parametrize("n_in", [512, 4096, 11008, 10500, 5120], ids=lambda n: "in%d" % n)
+def test_tiny_and_huge_gradients_take_the_exact_division(ops, oracle, n_in):
     # rows whose gradients leave the range of the reciprocal-based division (denormal and
-    # 1e-30 entries next to ordinary ones; a row with a 1e25 entry) must still be bit-exact
-    n_out, n_in, C = 8, 512, 11
+    # 1e-30 entries next to ordinary ones; a row with a 1e25 entry) must still be bit-exact, and so
+    # must rows with exact zeros, which hide the row's smallest magnitude from the cheap test --
+    # in the one-wave kernels, the cooperating-wave kernel (11008, 10500) and the two-pass one
+    n_out, C = 10, 11
     _, state, G, scale, v = synth.counter_case(31, n_out, n_in, C, oracle=oracle)
     G[0, ::3] = 1e-42
     G[1, ::5] = -3e-31
@@ -155,6 +158,11 @@ def test_tiny_and_huge_gradients_take_the_exact_division(ops, oracle):
     G[3] *= 1e-20
     G[4] = 0.0
     G[5, ::2] = 0.0
+    G[6, n_in - 1] = 0.0          # a single zero in the last wave's share
+    G[7, ::7] = 0.0
+    G[7, n_in // 2 + 1] = 1e-30   # zeros and a value too small for the reciprocal-based division
+    G[8, 3] = 0.0
+    G[8, n_in - 2] = -1e-41
     d = [dev(state), dev(scale), dev(v)]
     ops.apply_update_dense(*d, dev(G), C, 0.5, 0.0, 0.9, 0.0, 99)
     assert_bit_exact([host(t) for t in d], oracle.update_dense(state, scale, v, G, C, 0.5, 0.0, 0.9, 0.0, 99))
