@@ -142,3 +142,30 @@ def test_batched_updates_reject_a_state_listed_twice_and_validate_every_tensor_f
             assert L.mcc_last_error().decode().startswith("tensor 1:")
         finally:
             L.mcc_set_contraction_mode(0)
+
+
+def test_package_fails_loudly_without_the_library():
+    # no CPU path stands in for the HIP library: with the shared object missing, loading raises
+    import subprocess
+    import sys
+    code = (
+        "import motifcl_amd\n"
+        "from motifcl_amd.lib import LibraryMissing\n"
+        "try:\n"
+        "    motifcl_amd.load()\n"
+        "except LibraryMissing as e:\n"
+        "    print('missing:', e)\n"
+        "else:\n"
+        "    raise SystemExit('loaded something')\n"
+        "from motifcl_amd import ops\n"
+        "try:\n"
+        "    ops.fused_workspace_nbytes(8, 8, 8)\n"
+        "except LibraryMissing:\n"
+        "    print('op raised')\n"
+        "else:\n"
+        "    raise SystemExit('op answered without the library')\n"
+    )
+    env = dict(os.environ, MOTIFCL_AMD_LIB="/nonexistent/libmotifcl_amd.so")
+    out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "missing:" in out.stdout and "op raised" in out.stdout
