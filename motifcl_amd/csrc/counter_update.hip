@@ -61,6 +61,15 @@ __device__ __forceinline__ void build_luts(Luts& l, const Codec& cd, const LutGe
     __syncthreads();
 }
 
+// A gradient element is read exactly once by the register-resident kernels: a non-temporal load
+// keeps it from displacing the state words (whose overlapping 4-byte loads do want the cache) and
+// measured +1.8 % on 4096-wide rows.  State loads and stores gained nothing from the hint.
+__device__ __forceinline__ float4 load_grad4_once(const float4* p) {
+    typedef float f4v __attribute__((ext_vector_type(4)));
+    const f4v v = __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+
 // Byte-granular access to one packed group (any alignment, any position).
 __device__ __forceinline__ uint32_t load_group(const uint8_t* p) {
     return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
@@ -272,7 +281,7 @@ __device__ __forceinline__ void load_row(const UpdateTensor& t, int row, int lan
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const uint32_t gc = j < kLast ? (uint32_t)lane + kWave * j : gc_last;
-        q[j] = g_row[gc];
+        q[j] = load_grad4_once(g_row + gc);
         // only the row's last iteration can hold the tensor's last group
         w[j] = j < kLast ? load_group_dword(s_row + 3u * gc)
                          : load_group_dword_or_tail(s_row + 3u * gc, last_row && gc == gpr - 1);
@@ -410,7 +419,7 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
         for (int j = 0; j < kChunk; ++j) {
             const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j);
             const uint32_t gc = gi < gpr ? gi : gpr - 1;
-            q[j] = g_row[gc];
+            q[j] = load_grad4_once(g_row + gc);
             w[j] = load_row_word(s_row, gc, gpr, last_row);
         }
 #pragma unroll
@@ -522,7 +531,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
         for (int jj = 0; jj < J; ++jj) {
             const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
             const uint32_t gc = gi < gpr ? gi : gpr - 1;
-            q[jj] = g_row[gc];
+            q[jj] = load_grad4_once(g_row + gc);
             words[jj] = load_row_word(s_row, gc, gpr, last_row);
         }
         // What does not depend on the order happens before the hand-off, in all waves at once: the
