@@ -82,3 +82,22 @@ def test_plain_contraction_uses_spans_and_matches(ops, spans_mode):
     assert torch.equal(c1, c2)
     want = a.double().t() @ b.double()
     assert float((c1.double() - want).abs().max() / want.abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("tokens", [16, 32, 48, 64, 80, 96, 112, 128, 144, 272])
+def test_wide_tiles_with_few_slabs_match_the_small_tiles(ops, tokens):
+    """The 256 x 256 tile loop keeps four 16-token slabs in flight and runs four slabs per
+    iteration; token counts below and around that depth must give the bits of the 128 x 128 tiles,
+    which a 4096 x 2048 product (half a round of wide tiles) still uses."""
+    m = n = 4096
+    a = ops.fill_normal(torch.empty(tokens, m, device="cuda"), 31, 0.01)
+    b = ops.fill_normal(torch.empty(tokens, n, device="cuda"), 32, 1.0)
+    c = torch.empty(m, n, device="cuda")
+    ops.matmul_transpose_a(a, b, c)
+    for half in range(2):
+        bh = b[:, half * 2048:(half + 1) * 2048].contiguous()
+        ch = torch.empty(m, 2048, device="cuda")
+        ops.matmul_transpose_a(a, bh, ch)
+        assert torch.equal(c[:, half * 2048:(half + 1) * 2048], ch)
+    want = a.double().t() @ b.double()
+    assert float((c.double() - want).abs().max() / want.abs().max()) < 1e-5
