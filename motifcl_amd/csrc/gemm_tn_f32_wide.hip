@@ -1,6 +1,6 @@
 // The weight-gradient contraction c[m,n] = sum_k a[k,m] * b[k,n] on the fp32 matrix cores with
 // 256 x 256 tiles: 8 waves (2 down x 4 across, 128 x 64 each), slabs of 16 tokens copied straight
-// into one of two LDS buffers (global_load_lds_dwordx4).  Against the 128 x 128 tiles of
+// into one of four LDS buffers (global_load_lds_dwordx4).  Against the 128 x 128 tiles of
 // gemm_tn_f32.hip a workgroup copies half as many operand bytes per flop.  Every output element
 // still accumulates its tokens in the same order, two at a time, so the result is the same bits.
 // Whole tiles and whole slabs only.
@@ -8,12 +8,8 @@
 // Operand reads.  v_mfma_f32_32x32x2_f32 takes one float per lane from each operand; which matrix
 // row a lane's float belongs to is the kernel's choice.  Here lane l of the wave's four 32-row
 // blocks supplies rows 4 l .. 4 l + 3 (one per block) and columns 2 l, 2 l + 1, so a step's six
-// operand floats are one 16-byte and one 8-byte LDS read instead of six 4-byte ones (+2.7 % on
-// 4096 x 4096 at 32768 tokens: 92 % instead of 90 % of the peak at the measured clock); the
-// accumulators then hold a permuted tile, which the stores undo.  The reads are written as
-// float loads that the compiler merges: a read through a float4 / float2 pointer carries no
-// type-based alias information and makes the compiler wait for the copies of the next slab
-// (s_waitcnt vmcnt(0)) before every first read of a slab, which costs 9 %.
+// operand floats are one 16-byte and one 8-byte LDS read instead of six 4-byte ones; the
+// accumulators then hold a permuted tile, which the stores undo.
 //
 // Shapes of more than two rounds of tiles that are not whole rounds (11008 x 4096: 688 tiles on
 // 256 CUs) run as one launch of one workgroup per CU in which every workgroup gets the same number
@@ -73,8 +69,8 @@ __device__ __forceinline__ void wide_zero(WideAcc& acc) {
 // begins with a barrier followed by a full LDS latency with the matrix pipes idle, and the copies
 // of the next slab are issued between two slabs by both waves of a SIMD at the same moment, whose
 // address arithmetic leaves the matrix pipe idle.  Measured on 4096 x 4096 at 32768 tokens: the
-// compiler's loop 91.8 % of the peak; matrix instructions, operand reads and barriers alone
-// 98.5 %; this loop 94-95 %.
+// compiler's loop 91.8 % of the peak; matrix instructions, operand reads and barriers alone (no
+// copies, no operands from memory) 98.5 %; this loop 96.6 %, and 98 % with its copies left out.
 //
 // Registers.  A step's operands sit in fixed registers -- set 0 in v[232:235] (a) and v[240:241]
 // (b), set 1 in v[236:239] and v[242:243] -- because an assembly operand cannot name one register
@@ -102,58 +98,78 @@ __device__ __forceinline__ void wide_zero(WideAcc& acc) {
     "ds_read_b128 v[236:239], " VA " offset:" #BUF "+2048*" #STEP "\n" \
     "ds_read_b64 v[242:243], " VB " offset:" #BUF "+16384+2048*" #STEP "\n"
 #define MCC_WIDE_AHEAD "s_waitcnt lgkmcnt(2)\n"  // all reads but the two just issued have returned
+// A step's matrix instructions with two of the wave's copies in their shadow: 16 bytes per lane
+// from the addresses in P0 and P1 to the LDS addresses dst + D0 and dst + D1.
+#define MCC_WIDE_MFMA8_COPY(A0, A1, A2, A3, B0, B1, D0, P0, D1, P1)          \
+    "s_add_u32 m0, %[dst], " #D0 "\n"                                        \
+    MCC_WIDE_MFMA("c00", A0, B0)                                             \
+    "global_load_lds_dwordx4 " P0 ", off\n"                                  \
+    "s_add_u32 m0, %[dst], " #D1 "\n"                                        \
+    MCC_WIDE_MFMA("c01", A0, B1) MCC_WIDE_MFMA("c10", A1, B0)                \
+    "global_load_lds_dwordx4 " P1 ", off\n"                                  \
+    MCC_WIDE_MFMA("c11", A1, B1) MCC_WIDE_MFMA("c20", A2, B0) MCC_WIDE_MFMA("c21", A2, B1) \
+    MCC_WIDE_MFMA("c30", A3, B0) MCC_WIDE_MFMA("c31", A3, B1)
+#define MCC_WIDE_USE0_COPY(D0, P0, D1, P1) MCC_WIDE_MFMA8_COPY("v232", "v233", "v234", "v235", "v240", "v241", D0, P0, D1, P1)
+#define MCC_WIDE_USE1_COPY(D0, P0, D1, P1) MCC_WIDE_MFMA8_COPY("v236", "v237", "v238", "v239", "v242", "v243", D0, P0, D1, P1)
+// USE (a set's eight matrix instructions), with the two copies if this wave's turn (%[go]) is TURN
+#define MCC_WIDE_USE_OR_COPY(ID, K, TURN, USE, USE_COPY)                  \
+    "s_cmp_eq_u32 %[go], " #TURN "\n"                                     \
+    "s_cbranch_scc0 .Lmcc_wide_plain" #ID #K "_%=\n"                      \
+    USE_COPY                                                              \
+    "s_branch .Lmcc_wide_join" #ID #K "_%=\n"                             \
+    ".Lmcc_wide_plain" #ID #K "_%=:\n"                                    \
+    USE                                                                   \
+    ".Lmcc_wide_join" #ID #K "_%=:\n"
 // One slab out of the buffer (VA, VB, BUF); the next one is in (VAN, VBN, BUFN), and DST is the
-// byte offset of the buffer that held the slab before this one.  On entry the reads of step 0 are
-// in flight (set 0); every step first issues the reads of the step after it into the other set
-// and then waits for its own, so a wave never waits for a read it has only just issued.  Before
-// the last step every wave waits for its copies of the next slab (the four of the slab after
-// that may stay in flight, if there is one) and for the other waves; the last step's read-ahead
-// is step 0 of the next slab.  That barrier also says that nobody reads the slab before this one
-// any more, so -- if there is a slab three ahead -- the last step issues the wave's four copies of
-// it into that buffer (rows wave and wave + 8 of a from pa0 and pa1, of b from pb0 and pb1, to
-// LDS address dst + DST + 0, 8, 16, 24 KiB), each in the shadow of a matrix instruction.
+// byte offset of the buffer three on, which held the slab before this one.  On entry the reads
+// of step 0 are in flight (set 0); every step first issues the reads of the step after it into
+// the other set and then waits for its own, so a wave never waits for a read it has only just
+// issued.  Before the last step every wave waits for its own reads, for its copies of the next
+// slab (those of the two slabs after it may stay in flight) and for the other waves; the last
+// step's read-ahead is step 0 of the next slab.  The barrier therefore also says that nobody
+// reads this slab's buffer any more, and the next slab may fill it: if there is a slab three
+// ahead, the wave issues its four copies of it (rows wave and wave + 8 of a from pa0 and pa1, of
+// b from pb0 and pb1, to LDS address dst + DST + 0, 8, 16, 24 KiB) in the first four steps, each
+// in the shadow of a matrix instruction.  The copy unit takes a few dozen cycles per instruction
+// and a wave that waits for it issues nothing else, so the two waves of a SIMD take turns: waves
+// 0-3 copy in steps 0 and 2, waves 4-7 in steps 1 and 3 (%[ph]), and the matrix pipe always has
+// one wave that is not copying.  (All eight waves copying in the same step: 1 % slower; copies
+// between the slabs, outside the matrix instructions: 3 % slower.)
 #define MCC_WIDE_SLAB(ID, VA, VB, BUF, VAN, VBN, BUFN, DST)                            \
-    MCC_WIDE_READ1(VA, VB, BUF, 1) MCC_WIDE_AHEAD MCC_WIDE_USE0                        \
-    MCC_WIDE_READ0(VA, VB, BUF, 2) MCC_WIDE_AHEAD MCC_WIDE_USE1                        \
-    MCC_WIDE_READ1(VA, VB, BUF, 3) MCC_WIDE_AHEAD MCC_WIDE_USE0                        \
-    MCC_WIDE_READ0(VA, VB, BUF, 4) MCC_WIDE_AHEAD MCC_WIDE_USE1                        \
-    MCC_WIDE_READ1(VA, VB, BUF, 5) MCC_WIDE_AHEAD MCC_WIDE_USE0                        \
-    MCC_WIDE_READ0(VA, VB, BUF, 6) MCC_WIDE_AHEAD MCC_WIDE_USE1                        \
-    MCC_WIDE_READ1(VA, VB, BUF, 7) MCC_WIDE_AHEAD MCC_WIDE_USE0                        \
-    "s_add_u32 %[t], %[i], 2\n"                                                        \
-    "s_cmp_lt_u32 %[t], %[n]\n"                                                        \
-    "s_cbranch_scc0 .Lmcc_wide_tail" #ID "_%=\n"                                       \
-    "s_waitcnt vmcnt(4)\n"                                                             \
-    "s_branch .Lmcc_wide_landed" #ID "_%=\n"                                           \
-    ".Lmcc_wide_tail" #ID "_%=:\n"                                                     \
-    "s_waitcnt vmcnt(0)\n"                                                             \
-    ".Lmcc_wide_landed" #ID "_%=:\n"                                                   \
-    "s_barrier\n"                                                                      \
-    MCC_WIDE_READ0(VAN, VBN, BUFN, 0) MCC_WIDE_AHEAD                                   \
     "s_add_u32 %[t], %[i], 3\n"                                                        \
     "s_cmp_lt_u32 %[t], %[n]\n"                                                        \
-    "s_cbranch_scc0 .Lmcc_wide_last" #ID "_%=\n"                                       \
-    "s_add_u32 m0, %[dst], " #DST "\n"                                                 \
-    MCC_WIDE_MFMA("c00", "v236", "v242")                                               \
-    "global_load_lds_dwordx4 %[pa0], off\n"                                            \
-    "s_add_u32 m0, %[dst], " #DST "+0x2000\n"                                          \
-    MCC_WIDE_MFMA("c01", "v236", "v243") MCC_WIDE_MFMA("c10", "v237", "v242")          \
-    "global_load_lds_dwordx4 %[pa1], off\n"                                            \
-    "s_add_u32 m0, %[dst], " #DST "+0x4000\n"                                          \
-    MCC_WIDE_MFMA("c11", "v237", "v243") MCC_WIDE_MFMA("c20", "v238", "v242")          \
-    "global_load_lds_dwordx4 %[pb0], off\n"                                            \
-    "s_add_u32 m0, %[dst], " #DST "+0x6000\n"                                          \
-    MCC_WIDE_MFMA("c21", "v238", "v243") MCC_WIDE_MFMA("c30", "v239", "v242")          \
-    "global_load_lds_dwordx4 %[pb1], off\n"                                            \
-    MCC_WIDE_MFMA("c31", "v239", "v243")                                               \
+    "s_cselect_b32 %[go], %[ph], 2\n"                                                  \
+    MCC_WIDE_READ1(VA, VB, BUF, 1) MCC_WIDE_AHEAD                                      \
+    MCC_WIDE_USE_OR_COPY(ID, 0, 0, MCC_WIDE_USE0, MCC_WIDE_USE0_COPY(DST, "%[pa0]", DST+0x2000, "%[pa1]")) \
+    MCC_WIDE_READ0(VA, VB, BUF, 2) MCC_WIDE_AHEAD                                      \
+    MCC_WIDE_USE_OR_COPY(ID, 1, 1, MCC_WIDE_USE1, MCC_WIDE_USE1_COPY(DST, "%[pa0]", DST+0x2000, "%[pa1]")) \
+    MCC_WIDE_READ1(VA, VB, BUF, 3) MCC_WIDE_AHEAD                                      \
+    MCC_WIDE_USE_OR_COPY(ID, 2, 0, MCC_WIDE_USE0, MCC_WIDE_USE0_COPY(DST+0x4000, "%[pb0]", DST+0x6000, "%[pb1]")) \
+    MCC_WIDE_READ0(VA, VB, BUF, 4) MCC_WIDE_AHEAD                                      \
+    MCC_WIDE_USE_OR_COPY(ID, 3, 1, MCC_WIDE_USE1, MCC_WIDE_USE1_COPY(DST+0x4000, "%[pb0]", DST+0x6000, "%[pb1]")) \
     "v_lshl_add_u64 %[pa0], %[pa0], 0, %[sa]\n"                                        \
     "v_lshl_add_u64 %[pa1], %[pa1], 0, %[sa]\n"                                        \
     "v_lshl_add_u64 %[pb0], %[pb0], 0, %[sb]\n"                                        \
     "v_lshl_add_u64 %[pb1], %[pb1], 0, %[sb]\n"                                        \
-    "s_branch .Lmcc_wide_next" #ID "_%=\n"                                             \
-    ".Lmcc_wide_last" #ID "_%=:\n"                                                     \
+    MCC_WIDE_READ1(VA, VB, BUF, 5) MCC_WIDE_AHEAD MCC_WIDE_USE0                        \
+    MCC_WIDE_READ0(VA, VB, BUF, 6) MCC_WIDE_AHEAD MCC_WIDE_USE1                        \
+    MCC_WIDE_READ1(VA, VB, BUF, 7) MCC_WIDE_AHEAD MCC_WIDE_USE0                        \
+    "s_cmp_lt_u32 %[t], %[n]\n"                                                        \
+    "s_cbranch_scc0 .Lmcc_wide_two" #ID "_%=\n"                                        \
+    "s_waitcnt vmcnt(8) lgkmcnt(0)\n"                                                  \
+    "s_branch .Lmcc_wide_landed" #ID "_%=\n"                                           \
+    ".Lmcc_wide_two" #ID "_%=:\n"                                                      \
+    "s_add_u32 %[t], %[i], 2\n"                                                        \
+    "s_cmp_lt_u32 %[t], %[n]\n"                                                        \
+    "s_cbranch_scc0 .Lmcc_wide_one" #ID "_%=\n"                                        \
+    "s_waitcnt vmcnt(4) lgkmcnt(0)\n"                                                  \
+    "s_branch .Lmcc_wide_landed" #ID "_%=\n"                                           \
+    ".Lmcc_wide_one" #ID "_%=:\n"                                                      \
+    "s_waitcnt vmcnt(0) lgkmcnt(0)\n"                                                  \
+    ".Lmcc_wide_landed" #ID "_%=:\n"                                                   \
+    "s_barrier\n"                                                                      \
+    MCC_WIDE_READ0(VAN, VBN, BUFN, 0)                                                  \
     MCC_WIDE_USE1                                                                      \
-    ".Lmcc_wide_next" #ID "_%=:\n"                                                     \
     "s_add_u32 %[i], %[i], 1\n"                                                        \
     "s_cmp_lt_u32 %[i], %[n]\n"
 
@@ -163,8 +179,8 @@ __device__ __forceinline__ void wide_zero(WideAcc& acc) {
 // read.
 //
 // LDS holds kWideBuffers = 4 slabs.  The barrier of slab s says that slab s + 1 has landed and
-// that nobody reads slab s - 1 any more, so the copies of slab s + 3 go into that buffer right
-// after it and have almost three slabs' time to land.  Buffers 0 and 1 are addressed from one
+// that nobody reads slab s any more, so the copies of slab s + 4 go into that buffer during the
+// first steps of slab s + 1 and have two and a half slabs' time to land.  Buffers 0 and 1 are addressed from one
 // pair of address registers, 2 and 3 from another 64 KiB on (the offset field of an LDS read has
 // 16 bits), so the loop body is four slabs with constant offsets and the per-slab work outside
 // the matrix instructions is a handful of scalar instructions.
@@ -202,7 +218,8 @@ __device__ __forceinline__ void wide_accumulate(const float* __restrict__ a, con
     uint64_t pa0 = (uint64_t)a_next, pa1 = (uint64_t)(a_next + (size_t)8 * M);
     uint64_t pb0 = (uint64_t)b_next, pb1 = (uint64_t)(b_next + (size_t)8 * N);
     const uint64_t sa = (uint64_t)kBK * (uint64_t)M * 4u, sb = (uint64_t)kBK * (uint64_t)N * 4u;
-    int i, tmp;
+    const int turn = __builtin_amdgcn_readfirstlane(t.wave >> 2);
+    int i, tmp, go;
     asm volatile(
         "s_mov_b32 %[i], 0\n"
         MCC_WIDE_READ0("%[va]", "%[vb]", 0, 0)
@@ -223,9 +240,9 @@ __device__ __forceinline__ void wide_accumulate(const float* __restrict__ a, con
         "s_nop 7\n"
         : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]),
           [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [pa0] "+v"(pa0),
-          [pa1] "+v"(pa1), [pb0] "+v"(pb0), [pb1] "+v"(pb1), [i] "=&s"(i), [t] "=&s"(tmp)
+          [pa1] "+v"(pa1), [pb0] "+v"(pb0), [pb1] "+v"(pb1), [i] "=&s"(i), [t] "=&s"(tmp), [go] "=&s"(go)
         : [va] "v"(va), [vb] "v"(vb), [va2] "v"(va + 65536u), [vb2] "v"(vb + 65536u), [n] "s"(slabs), [dst] "s"(dst),
-          [sa] "s"(sa), [sb] "s"(sb)
+          [sa] "s"(sa), [sb] "s"(sb), [ph] "s"(turn)
         // and m0, which the compiler sets before each of its own uses
         : "memory", "scc", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242",
           "v243");

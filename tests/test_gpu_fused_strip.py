@@ -167,6 +167,7 @@ def test_second_strip_step_on_another_stream_is_refused_while_the_first_runs(ops
     # everything the second call touches exists before the first is launched: an allocation in
     # between may wait for the device, and the first step would be over before the second is tried
     state2, scale2, v2 = state.clone(), scale.clone(), v.clone()
+    busy = state.clone(), scale.clone(), v.clone()
     x = torch.randn(n, n_in, device="cuda")
     dy = torch.randn(n, n_out, device="cuda") * 0.01
     nbytes = ops.fused_strip_workspace_nbytes(n_in, n_out, n)
@@ -174,13 +175,19 @@ def test_second_strip_step_on_another_stream_is_refused_while_the_first_runs(ops
     ws2 = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     side = torch.cuda.Stream()
     torch.cuda.synchronize()
-    ops.apply_update_fused(state, scale, v, dy, x, ws1, C, 3e-3, 0.0, 0.9, 1e-3, 1)  # about 4.5 ms of work
+    # several steps in a row (about 4.5 ms each) keep the device busy well beyond the host's way to
+    # the second call, whatever the host is doing in between
+    for _ in range(6):
+        ops.apply_update_fused(*busy, dy, x, ws1, C, 3e-3, 0.0, 0.9, 1e-3, 1)
     with torch.cuda.stream(side):
         with pytest.raises(MccError, match="different stream"):
             ops.apply_update_fused(state2, scale2, v2, dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
     torch.cuda.synchronize()
     ops.fused_check(ws1, n_in, n_out, n)
-    # once the first has finished the other stream may go
+    # once the first stream's steps have finished the other stream may go
+    ops.apply_update_fused(state, scale, v, dy, x, ws1, C, 3e-3, 0.0, 0.9, 1e-3, 1)
+    torch.cuda.synchronize()
+    ops.fused_check(ws1, n_in, n_out, n)
     with torch.cuda.stream(side):
         ops.apply_update_fused(state2, scale2, v2, dy, x, ws2, C, 3e-3, 0.0, 0.9, 1e-3, 1)
     torch.cuda.synchronize()
