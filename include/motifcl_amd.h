@@ -241,7 +241,7 @@ int mcc_compact_counter_apply_update_fused_batched(
  *   MCC_CONTRACTION_BF16X6  both operands split into three bf16 terms, six bf16
  *                           matrix passes per product: per-product error of one
  *                           binary32 rounding, as the fp32 instruction, at about
- *                           1.3 x its speed on 7B-sized layers (71 against 93 ms
+ *                           1.2 x its speed on 7B-sized layers (72 against 88 ms
  *                           for a seven-tensor layer step at 32768 tokens).  Used
  *                           for whole 128 x 128 tiles and
  *                           token counts that are multiples of 32; other shapes
