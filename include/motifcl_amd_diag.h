@@ -25,6 +25,15 @@ extern "C" {
 void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
 
 /*
+ * Tiles of the strip-workspace step: 0 (default) chosen by shape -- 256 x 256
+ * tiles where whole rounds of them keep the device busy, 128 x 128 otherwise --,
+ * 1 the 256 x 256 tiles whenever the shape allows them (sides multiples of 256,
+ * token count a multiple of 16, 16-byte aligned operands), 2 never.  Both kernels
+ * write the same bytes; tests use the switch to compare them on small shapes.
+ */
+void mcc_compact_counter_fused_strip_set_tile_mode(int mode);
+
+/*
  * The contraction of shapes that are more than two but not a whole number of rounds of
  * 256 x 256 tiles runs as one launch in which neighbouring workgroups hand a partly
  * summed tile on through the output buffer; a workgroup that does not find the tile it

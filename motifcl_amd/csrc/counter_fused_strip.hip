@@ -35,6 +35,7 @@
 
 #include "counter_math.hpp"
 #include "gemm_tile.hpp"
+#include "gemm_wide_tile.hpp"
 #include "launch.hpp"
 #include "wave_ops.hpp"
 
@@ -184,10 +185,10 @@ __device__ __forceinline__ int give_up(const StripArgs& a, StripControl* c) {
 }
 
 // Thread 0 polls until *word >= want (a hand-off counter) or, with DECISION, until *word != 0,
-// the status word is raised, or the spin budget is spent; e.ok tells the workgroup whether the
-// condition came true.  All threads of the workgroup call it.
+// the status word is raised, or the spin budget is spent; ok_word (in LDS) tells the workgroup
+// whether the condition came true.  All threads of the workgroup call it.
 template <bool DECISION>
-__device__ __forceinline__ bool wait_for(const StripArgs& a, const int* word, int want, EpilogueLds& e) {
+__device__ __forceinline__ bool wait_for(const StripArgs& a, const int* word, int want, int& ok_word) {
     if (threadIdx.x == 0) {
         int ok = 1;
         unsigned spins = 0, polls = 0;
@@ -207,11 +208,11 @@ __device__ __forceinline__ bool wait_for(const StripArgs& a, const int* word, in
                 break;
             }
         }
-        e.ok = ok;
+        ok_word = ok;
     }
     __syncthreads();
-    const bool ok = e.ok != 0;
-    __syncthreads();  // e.ok may be rewritten by the next wait
+    const bool ok = ok_word != 0;
+    __syncthreads();  // the word may be rewritten by the next wait
     return ok;
 }
 
@@ -319,7 +320,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         // ---- chain hand-off: step `step` of chains 32*parity .. 32*parity+31 -------------
         // The 128 x 32 chain block (16 KiB per sum) is staged in the contraction's LDS slab buffer,
         // which is free by now; each thread moves 16 floats, 256 contiguous bytes per wave and access.
-        if (!wait_for<false>(a, &control->published[parity], step, e)) {
+        if (!wait_for<false>(a, &control->published[parity], step, e.ok)) {
             if (threadIdx.x == 0) give_up(a, control);
             return;
         }
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         park_accumulators(acc);
         tp = fresh_tile_pos();
         lane = tp.tid & 63, wave = tp.tid >> 6;
-        bool committed = wait_for<true>(a, &control->decision, 0, e);
+        bool committed = wait_for<true>(a, &control->decision, 0, e.ok);
         if (tp.tid == 0) {
             int d = committed ? load_relaxed(&control->decision) : give_up(a, control);
             if (d < 0 && committed) give_up(a, control);  // aborted by another tile: count this launch as failed
@@ -464,6 +465,229 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
     }
 }
 
+// ------------------------------------------------------------------------------ wide tiles
+// The same step on the 256 x 256 tiles of gemm_wide_tile.hpp, one workgroup per CU.  A strip is 256
+// rows and a tile covers 64 consecutive packed groups of its rows -- one step of all 64 chains --
+// so the tiles of a strip form a single hand-off sequence: tile ct waits for tile ct - 1.  In the
+// permuted accumulator layout a lane holds two neighbouring columns of each of its 64 rows, so a
+// packed group is a pair of lanes: the even lane adds elements 0 and 1 to the chain value, hands
+// the sum to the odd lane (DPP), which adds elements 2 and 3 and stores it; the four adds are the
+// reference's, in its order.  Chain values go straight between registers and the chain block
+// (device-scope atomic accesses, 64 contiguous bytes per 16 lanes).  A wide strip uses the chain
+// storage and the first control block of the two 128-row strips it covers, so the workspace is
+// the same for both kernels.
+constexpr int kWideChainSetFloats = kWide * 64;  // 256 rows x 64 chains
+static_assert(2 * kWideChainSetFloats == 2 * kStripChainFloats, "a wide strip takes the room of two 128-row strips");
+
+struct WideEpilogueLds {
+    int q_off[64];
+    float c_f[64];
+    float dn[kWide];     // denominator of each row of the strip
+    float k[kWide];      // Cf / scale_new
+    float ratio[kWide];  // scale_old / scale_new
+    uint8_t fin[kLutFinMaxBytes];
+    int ok;
+};
+
+// Value of the even lane of the calling lane's pair (lanes 2 n and 2 n + 1).
+__device__ __forceinline__ float from_even_lane(float x) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), 0xa0, 0xf, 0xf, false));  // quad_perm:[0,0,2,2]
+}
+// OR over the two lanes of each pair.
+__device__ __forceinline__ uint32_t pair_or(uint32_t x) {
+    return x | (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xb1, 0xf, 0xf, false);  // quad_perm:[1,0,3,2]
+}
+
+template <bool WITH_GS>
+MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
+    __shared__ __attribute__((aligned(1024))) float lds[kWideBuffers * kWideSlabFloats];
+    __shared__ WideEpilogueLds e;
+    const WideLane t = wide_lane();
+    for (int i = t.tid; i < 64; i += kWideThreads) {
+        e.q_off[i] = q_off_entry((uint32_t)i, a.cd, a.geom);
+        e.c_f[i] = (float)code_c((uint32_t)i, a.cd);
+    }
+    for (int i = t.tid, n = fin_size(a.geom); i < n; i += kWideThreads) fill_fin_entry(i, a.cd, a.geom, e.fin);
+    __syncthreads();
+
+    const int groups_per_row = a.in_features >> 2;
+    const uint32_t last_group_off = 3u * ((uint32_t)a.out_features * (uint32_t)groups_per_row - 1u);
+    const uint32_t row_bytes = 3u * (uint32_t)groups_per_row;
+    const int pair_half = t.l32 & 1;                       // 0: elements 0, 1 of the packed group; 1: elements 2, 3
+    const int slot = (t.wn0 >> 2) + (t.l32 >> 1);          // the group's place in the tile = its chain
+    // accumulator (i, j, r) is row row0 + 32 (r / 4) + 4 (r % 4) + i, column 4 slot + 2 pair_half + j of the tile
+    const int row0 = t.wm0 + 16 * t.half;
+    auto row_of = [&](int i, int r) { return row0 + 32 * (r / 4) + 4 * (r % 4) + i; };
+
+    for (int tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
+        // once a workgroup has given up nothing new is started: a strip whose tiles have not all
+        // published cannot have been committed, and this tile has not published yet
+        if (t.tid == 0) e.ok = load_relaxed(a.status) == 0 ? 1 : 0;
+        __syncthreads();
+        const bool healthy = e.ok != 0;
+        __syncthreads();
+        if (!healthy) return;
+        const int strip = tile / a.tiles_per_strip;
+        const int ct = tile - strip * a.tiles_per_strip;
+        const int m0 = strip * kWide, n0 = ct * kWide;
+        StripControl* control = a.control + 2 * strip;
+        float* chain = a.chain + (size_t)strip * (2 * kWideChainSetFloats);
+
+        WideAcc acc;
+        wide_zero(acc);
+        wide_accumulate(a.grad_out + m0, a.x + n0, a.out_features, a.in_features, a.tokens, acc, lds, t);
+
+        // Old per-row values, read before anything of this strip is written: tile 0 overwrites
+        // them only after the strip has been committed, and commits happen after every tile of
+        // the strip has been here.
+        float s_old = 0.0f, v_old = 0.0f;
+        if (t.tid < kWide) {
+            s_old = a.scale[m0 + t.tid];
+            v_old = a.v[m0 + t.tid];
+        }
+        // byte offset of this lane's packed group in row row0 of the strip (the launch checks that
+        // the state is smaller than 2 GiB) and the element index of its first column there
+        const uint32_t my_state = (uint32_t)(m0 + row0) * row_bytes + 3u * (uint32_t)((n0 >> 2) + slot);
+        const uint32_t my_elem = (uint32_t)(m0 + row0) * (uint32_t)a.in_features +
+                                 (uint32_t)(n0 + 4 * slot + 2 * pair_half);
+        // One 4-byte load per lane and group; the tensor's last group has no byte after it, so it
+        // is fetched one byte early and shifted down.
+        auto load_word = [&](int i, int r) {
+            const uint32_t off = my_state + (uint32_t)(32 * (r / 4) + 4 * (r % 4) + i) * row_bytes;
+            const uint32_t is_last = off == last_group_off ? 1u : 0u;
+            uint32_t word;
+            __builtin_memcpy(&word, a.state + (off - is_last), 4);
+            return word >> (8 * is_last);
+        };
+
+        // ---- chain hand-off: step ct of all 64 chains of the strip's rows -------------------
+        if (!wait_for<false>(a, &control->published[0], ct, e.ok)) {
+            if (t.tid == 0) give_up(a, control);
+            return;
+        }
+#pragma unroll
+        for (int set = 0; set < (WITH_GS ? 2 : 1); ++set) {
+            float* my_chain = chain + set * kWideChainSetFloats + slot;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float in[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) in[r] = ct > 0 ? load_shared_f32(my_chain + row_of(i, r) * 64) : 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float v0, v1;
+                    if (set == 0) {
+                        v0 = acc[i][0][r] * acc[i][0][r];
+                        v1 = acc[i][1][r] * acc[i][1][r];
+                    } else {
+                        // g * t (kernels/compact_counter.cl:81-82): t from the element's code
+                        const uint32_t word = load_word(i, r) >> (12 * pair_half);
+                        v0 = acc[i][0][r] * (float)(code_q(word & 0x3fu, a.cd) - 1);
+                        v1 = acc[i][1][r] * (float)(code_q((word >> 6) & 0x3fu, a.cd) - 1);
+                    }
+                    const float first = (in[r] + v0) + v1;          // elements 0 and 1: the even lane's
+                    const float second = (from_even_lane(first) + v0) + v1;  // then 2 and 3: the odd lane's
+                    if (pair_half) store_shared_f32(my_chain + row_of(i, r) * 64, second);
+                }
+            }
+        }
+        stores_done();
+        __syncthreads();
+        if (t.tid == 0) {
+            __hip_atomic_store(&control->published[0], ct + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the last tile of the sequence commits the strip
+            if (ct + 1 == a.tiles_per_strip) {
+                __builtin_amdgcn_s_waitcnt(0);
+                cas_relaxed(&control->decision, 0, 1);
+            }
+        }
+
+        // ---- wait for the strip's decision ---------------------------------------------
+        bool committed = wait_for<true>(a, &control->decision, 0, e.ok);
+        if (t.tid == 0) {
+            int d = committed ? load_relaxed(&control->decision) : give_up(a, control);
+            if (d < 0 && committed) give_up(a, control);  // aborted by another tile: count this launch as failed
+            e.ok = d > 0 ? 1 : 0;
+        }
+        __syncthreads();
+        committed = e.ok != 0;
+        __syncthreads();
+        if (!committed) return;
+
+        // ---- row statistics: every tile finishes the rows of its strip itself ---------------
+        {
+            // wave w finishes rows 32 w .. 32 w + 31: lane l holds chain l of the row
+            constexpr int kRowsPerWave = kWide / 8;
+#pragma unroll
+            for (int set = 0; set < (WITH_GS ? 2 : 1); ++set) {
+                const float* mine = chain + set * kWideChainSetFloats + t.lane;
+                float part[kRowsPerWave];
+#pragma unroll
+                for (int rr = 0; rr < kRowsPerWave; ++rr)
+                    part[rr] = load_shared_f32(mine + (t.wave * kRowsPerWave + rr) * 64);
+#pragma unroll
+                for (int rr = 0; rr < kRowsPerWave; ++rr) {
+                    const float sum = tree_sum(part[rr], t.lane);
+                    if (t.lane == 0) (set == 0 ? e.dn : e.k)[t.wave * kRowsPerWave + rr] = sum;  // parked; replaced below
+                }
+            }
+        }
+        __syncthreads();
+        if (t.tid < kWide) {
+            const RowStats rs = finish_row_stats(e.dn[t.tid], WITH_GS ? e.k[t.tid] : 0.0f, v_old, s_old, a.in_features,
+                                                 WITH_GS ? a.lr_scale : 0.0f, a.rms_beta, a.rms_eps);
+            e.dn[t.tid] = rs.denom;
+            e.k[t.tid] = a.cd.Cf / rs.scale_new;
+            e.ratio[t.tid] = s_old / rs.scale_new;
+            if (ct == 0) {
+                a.v[m0 + t.tid] = rs.v_new;
+                a.scale[m0 + t.tid] = rs.scale_new;
+            }
+        }
+        __syncthreads();
+
+        // ---- ticks straight from the accumulators -----------------------------------------
+        TickConsts tc;
+        tc.r = 0.0f;
+        tc.neg_lr = -a.lr;
+        tc.neg_lim_neg = -(float)a.geom.lim_neg;
+        tc.lim_pos = (float)a.geom.lim_pos;
+        tc.two_m24 = 1.0f / 16777216.0f;
+        tc.seed_mix = seed_mix(a.seed);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // all 16 state loads are issued before the first tick
+            uint32_t word[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) word[r] = load_word(i, r);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = row_of(i, r);
+                tc.dn = e.dn[row];
+                tc.k = e.k[row];
+                const RebasedCounter c_reb{e.c_f, e.ratio[row]};
+                const uint32_t dr = (uint32_t)(32 * (r / 4) + 4 * (r % 4) + i);
+                const uint32_t elem = my_elem + dr * (uint32_t)a.in_features;
+                const uint32_t off = my_state + dr * row_bytes;
+                const uint32_t codes = word[r] >> (12 * pair_half);
+                const uint32_t nc0 = tick_code<false>(codes & 0x3fu, acc[i][0][r], tc, hash_first(elem), c_reb, e.q_off,
+                                                      e.fin);
+                const uint32_t nc1 = tick_code<false>((codes >> 6) & 0x3fu, acc[i][1][r], tc, hash_first(elem + 1u),
+                                                      c_reb, e.q_off, e.fin);
+                const uint32_t nw = pair_or((nc0 | (nc1 << 6)) << (12 * pair_half));
+                // bytes 0 and 1 of the group from the even lane, byte 2 from the odd one
+                if (pair_half) {
+                    a.state[off + 2] = (uint8_t)(nw >> 16);
+                } else {
+                    a.state[off] = (uint8_t)nw;
+                    a.state[off + 1] = (uint8_t)(nw >> 8);
+                }
+            }
+        }
+        __syncthreads();  // the row constants are rewritten by the next tile
+    }
+}
+
 __global__ void strip_clear_kernel(int* words, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) words[i] = 0;
@@ -513,6 +737,11 @@ DeviceState* current_device_state(hipError_t* err) {
 // seconds, far above any wait a healthy launch can see.
 constexpr unsigned kDefaultSpinLimit = 1u << 24;
 static std::atomic<unsigned> g_spin_limit{kDefaultSpinLimit};
+
+// Which tiles a strip launch uses: 0 the wide ones where they keep the device busy, 1 the wide ones
+// whenever the shape allows them, 2 never (tests compare the two kernels).
+static std::atomic<int> g_wide_mode{0};
+void set_fused_strip_wide_mode(int mode) { g_wide_mode.store(mode >= 0 && mode <= 2 ? mode : 0); }
 
 unsigned fused_strip_spin_limit() { return g_spin_limit.load(); }
 void set_fused_strip_spin_limit(unsigned spins) { g_spin_limit.store(spins ? spins : kDefaultSpinLimit); }
@@ -574,8 +803,10 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     // measured: with the rotating priority the direct-to-LDS main loop is 2 % slower here (it is
     // 3 % faster in the plain contraction), so the staged loop stays
     const bool gs = lr_scale != 0.0f;
-    auto kernel = vec_a ? (gs ? fused_strip_kernel<true, false, true> : fused_strip_kernel<true, false, false>)
-                        : (gs ? fused_strip_kernel<false, false, true> : fused_strip_kernel<false, false, false>);
+    typedef void (*StripKernel)(StripArgs);
+    StripKernel kernel = vec_a ? (gs ? fused_strip_kernel<true, false, true> : fused_strip_kernel<true, false, false>)
+                               : (gs ? fused_strip_kernel<false, false, true> : fused_strip_kernel<false, false, false>);
+    int threads = kGemmThreads;
 
     std::lock_guard<std::mutex> lock(g_mu);
     hipError_t err;
@@ -605,7 +836,33 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     if (err != hipSuccess) return err;
     err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
     if (err != hipSuccess) return err;
-    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kGemmThreads, 0);
+
+    // Wide tiles: whole 256 x 256 tiles, whole slabs, aligned operands -- and, unless forced, a shape
+    // whose strips come in rounds that keep at least four fifths of the CUs busy (4096 x 4096 is
+    // one round of 16 strips of 16 tiles, 11008 x 4096 three rounds for 2.69; 4096 x 11008 has 43
+    // tiles per strip, five strips per round and four rounds for 2.69, and stays on small tiles).
+    const int wide_mode = g_wide_mode.load();
+    if (wide_mode != 2 && vec_a && in_features % kWide == 0 && out_features % kWide == 0 && tokens >= kBK &&
+        tokens % kBK == 0) {
+        StripKernel wide = gs ? fused_strip_wide_kernel<true> : fused_strip_wide_kernel<false>;
+        int wide_per_cu = 0;
+        err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&wide_per_cu, wide, kWideThreads, 0);
+        if (err != hipSuccess) return err;
+        const long capacity = (long)cus * wide_per_cu;
+        const long tiles_x = in_features / kWide, wide_strips = out_features / kWide;
+        if (capacity >= tiles_x) {
+            const long per_round = capacity / tiles_x;
+            const long rounds = (wide_strips + per_round - 1) / per_round;
+            if (wide_mode == 1 || wide_strips * tiles_x * 5 >= rounds * capacity * 4) {
+                kernel = wide;
+                threads = kWideThreads;
+                a.tiles_per_strip = (int)tiles_x;
+                a.total_tiles = (int)(wide_strips * tiles_x);
+            }
+        }
+    }
+
+    err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0);
     if (err != hipSuccess) return err;
     const long capacity = (long)cus * per_cu;
     a.layer_wgs = cus;
@@ -620,7 +877,7 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
                        reinterpret_cast<int*>(ws), clear_words);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kGemmThreads), 0, stream, a);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), 0, stream, a);
     err = hipGetLastError();
     if (err != hipSuccess || capturing) return err;
     if (!dev->last_launch) {

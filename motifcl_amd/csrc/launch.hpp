@@ -97,13 +97,17 @@ hipError_t launch_gemm_tn_bf16x6(hipStream_t stream, const float* a, const float
                                  int k, int m, int n, const GemmTnPlan& plan);
 
 // Fused step that keeps G in the contraction's accumulators (counter_fused_strip.hip).
-// Shapes: in_features and out_features multiples of 128.
+// Shapes: in_features and out_features multiples of 128.  Large layers whose sides are multiples of
+// 256 run on 256 x 256 tiles (same workspace, same bytes).
 bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch);
 size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch);
 // Polls one device-side wait of the strip step may spend before it gives up (0 restores the
 // default, about four seconds; a test aid declared in motifcl_amd_diag.h).
 unsigned fused_strip_spin_limit();
 void set_fused_strip_spin_limit(unsigned spins);
+// Tiles of the strip step: 0 chosen by shape (256 x 256 where their rounds keep the device busy,
+// else 128 x 128), 1 wide whenever the shape allows, 2 never wide.  The result is the same bytes.
+void set_fused_strip_wide_mode(int mode);
 // *busy: another strip launch of this process is still running on a different stream of the GPU
 // (nothing was enqueued).  Strip launches that give up a wait raise a per-device count that
 // fused_strip_take_failures reads and clears (the stream must have been synchronised).

@@ -47,6 +47,43 @@ def run_both(ops, n, n_in, n_out, C, seed, lr=HP["lr"], lr_scale=HP["lr_scale"])
     return state, scale, v, x, dy, out
 
 
+@pytest.fixture()
+def tile_mode():
+    """Selects the strip step's tiles: 0 by shape, 1 the 256 x 256 tiles wherever possible, 2 never."""
+    import motifcl_amd
+    L = motifcl_amd.load()
+    yield L.mcc_compact_counter_fused_strip_set_tile_mode
+    L.mcc_compact_counter_fused_strip_set_tile_mode(0)
+
+
+# (N, in, out, C): sides that are multiples of 256 and whole 16-token slabs, which the wide tiles take
+WIDE_STRIP_SHAPES = [
+    (16, 256, 256, 11),     # one tile
+    (48, 512, 256, 3),      # one strip of two tiles, three slabs
+    (96, 1024, 512, 11),
+    (64, 768, 2048, 11),    # BASELINE cfg2 shapes, few tokens
+    (64, 2048, 768, 8),
+    (32, 4096, 4096, 11),   # one round of 16 strips of 16 tiles
+    (32, 4096, 2816, 11),   # 11 strips: one round that does not fill the device
+    (32, 11008, 1536, 11),  # 43 tiles per strip: five strips a round, two rounds
+]
+
+
+@pytest.mark.parametrize("lr_scale", [0.0, 0.05])
+@pytest.mark.parametrize("shape", WIDE_STRIP_SHAPES, ids=lambda s: "N%d_in%d_out%d_C%d" % s)
+def test_wide_strip_tiles_match_small_tiles_and_two_kernel_path(ops, tile_mode, shape, lr_scale):
+    n, n_in, n_out, C = shape
+    print("wide strip case", shape, lr_scale, flush=True)
+    tile_mode(2)
+    state, scale, v, _, _, (full, small) = run_both(ops, n, n_in, n_out, C, seed=n_in + n_out, lr_scale=lr_scale)
+    tile_mode(1)
+    _, _, _, _, _, (_, wide) = run_both(ops, n, n_in, n_out, C, seed=n_in + n_out, lr_scale=lr_scale)
+    assert not np.array_equal(full[0], state)
+    for a, b, c in zip(wide, small, full):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+        assert np.array_equal(a.view(np.uint8), c.view(np.uint8))
+
+
 @pytest.mark.parametrize("shape", STRIP_SHAPES, ids=lambda s: "N%d_in%d_out%d_C%d" % s)
 def test_strip_path_matches_two_kernel_path(ops, shape):
     n, n_in, n_out, C = shape
@@ -214,11 +251,14 @@ def test_two_strip_updates_in_a_row_are_deterministic(ops):
         assert np.array_equal(a, b)
 
 
-def test_given_up_wait_is_reported_and_leaves_whole_strips_untouched(ops):
+@pytest.mark.parametrize("wide", [False, True], ids=["tiles128", "tiles256"])
+def test_given_up_wait_is_reported_and_leaves_whole_strips_untouched(ops, tile_mode, wide):
     # a spin budget of one poll makes waits fail from the host side; the kernel must still drain,
     # the failure must surface through fused_check -- also after another layer has used the same
-    # workspace -- and every 128-row strip must be either fully updated or untouched
+    # workspace -- and every strip (128 or 256 rows) must be either fully updated or untouched
     import motifcl_amd
+    tile_mode(1 if wide else 2)
+    strip_rows = 256 if wide else 128
     from motifcl_amd.lib import MccError
     L = motifcl_amd.load()
     n, n_in, n_out, C = 32, 4096, 512, 11
@@ -248,14 +288,14 @@ def test_given_up_wait_is_reported_and_leaves_whole_strips_untouched(ops):
     got = [host(t) for t in d]
     row_bytes = n_in // 4 * 3
     untouched = 0
-    for s0 in range(0, n_out, 128):
-        rows = slice(s0, s0 + 128)
-        st = slice(s0 * row_bytes, (s0 + 128) * row_bytes)
+    for s0 in range(0, n_out, strip_rows):
+        rows = slice(s0, s0 + strip_rows)
+        st = slice(s0 * row_bytes, (s0 + strip_rows) * row_bytes)
         if np.array_equal(got[0][st], state[st]):
             untouched += 1
             assert np.array_equal(got[1][rows], scale[rows]) and np.array_equal(got[2][rows], v[rows])
         else:
-            assert np.array_equal(got[0][st], ref[0][st]), "strip %d is half-updated" % (s0 // 128)
+            assert np.array_equal(got[0][st], ref[0][st]), "strip %d is half-updated" % (s0 // strip_rows)
             assert np.array_equal(got[1][rows], ref[1][rows]) and np.array_equal(got[2][rows], ref[2][rows])
     assert untouched >= 1
     # with the default budget the same call completes and matches the two-kernel path
