@@ -30,8 +30,12 @@ void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
  * 1 the 256 x 256 tiles whenever the shape allows them (sides multiples of 256,
  * token count a multiple of 16, 16-byte aligned operands), 2 never.  Both kernels
  * write the same bytes; tests use the switch to compare them on small shapes.
+ * grid_cap > 0 holds the 256 x 256 kernel to that many workgroups, so that a
+ * small layer runs in several passes of its persistent grid and parks tiles
+ * whose strip ends in a later pass; the cap also enters the strip workspace
+ * size (the slots for parked tiles), so set it before sizing the workspace.  0 restores the device's own capacity.
  */
-void mcc_compact_counter_fused_strip_set_tile_mode(int mode);
+void mcc_compact_counter_fused_strip_set_tile_mode(int mode, int grid_cap);
 
 /*
  * The contraction of shapes that are more than two but not a whole number of rounds of

@@ -331,7 +331,7 @@ int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t 
         return fail(MCC_E_RUNTIME,
                     "compact-counter fused strip update gave up waiting for a neighbouring tile in " +
                         std::to_string(failures) + " launch(es) on this GPU since the last check; in such a launch "
-                        "whole 128-row strips of the tensor are left without their update (no strip is half-updated)");
+                        "whole strips of the tensor (128 or 256 rows) are left without their update (no strip is half-updated)");
     return MCC_OK;
 }
 

@@ -67,6 +67,8 @@ struct StripArgs {
     int* failures;          // the library's per-device count of strip launches' workgroups that gave up
     StripControl* control;  // [strip]
     float* chain;           // [strip][g^2, g*t][parity][128][32]
+    float* park;            // wide tiles: slots for tiles whose strip ends in a later pass (nullptr: none)
+    int park_first_wg;      // ... the first workgroup that has slots (two each)
     int tokens, in_features, out_features;
     int tiles_per_strip, total_tiles;
     int layer_wgs;  // workgroups the device takes in per residency layer (its CU count)
@@ -188,7 +190,8 @@ __device__ __forceinline__ int give_up(const StripArgs& a, StripControl* c) {
 // the status word is raised, or the spin budget is spent; ok_word (in LDS) tells the workgroup
 // whether the condition came true.  All threads of the workgroup call it.
 template <bool DECISION>
-__device__ __forceinline__ bool wait_for(const StripArgs& a, const int* word, int want, int& ok_word) {
+__device__ __forceinline__ bool wait_for(const StripArgs& a, const int* word, int want, int& ok_word,
+                                         int decision_naps = 0) {
     if (threadIdx.x == 0) {
         int ok = 1;
         unsigned spins = 0, polls = 0;
@@ -199,7 +202,7 @@ __device__ __forceinline__ bool wait_for(const StripArgs& a, const int* word, in
             // proportion to the hand-offs still to come instead of polling at full rate.  A
             // thousand workgroups polling a handful of words slow the contractions that are
             // still running by a third.
-            const int naps = DECISION ? 0 : (want - seen - 1) * kNapsPerHandOff;
+            const int naps = DECISION ? decision_naps : (want - seen - 1) * kNapsPerHandOff;
             __builtin_amdgcn_s_sleep(8);
             for (int n = 0; n < naps; ++n) __builtin_amdgcn_s_sleep(32);
             spins += 1u + (unsigned)naps;
@@ -498,6 +501,10 @@ __device__ __forceinline__ uint32_t pair_or(uint32_t x) {
     return x | (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xb1, 0xf, 0xf, false);  // quad_perm:[1,0,3,2]
 }
 
+// A parked tile: its 65536 accumulators in the order (register, thread), then the old scale and v of
+// the strip's 256 rows.  Only the workgroup that wrote a slot reads it, every thread its own values.
+constexpr int kParkSlotFloats = kWide * kWide + 2 * kWide;
+
 template <bool WITH_GS>
 MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
     __shared__ __attribute__((aligned(1024))) float lds[kWideBuffers * kWideSlabFloats];
@@ -519,91 +526,26 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
     const int row0 = t.wm0 + 16 * t.half;
     auto row_of = [&](int i, int r) { return row0 + 32 * (r / 4) + 4 * (r % 4) + i; };
 
-    for (int tile = blockIdx.x; tile < a.total_tiles; tile += gridDim.x) {
-        // once a workgroup has given up nothing new is started: a strip whose tiles have not all
-        // published cannot have been committed, and this tile has not published yet
-        if (t.tid == 0) e.ok = load_relaxed(a.status) == 0 ? 1 : 0;
-        __syncthreads();
-        const bool healthy = e.ok != 0;
-        __syncthreads();
-        if (!healthy) return;
-        const int strip = tile / a.tiles_per_strip;
-        const int ct = tile - strip * a.tiles_per_strip;
+    // One 4-byte load per lane and group; the tensor's last group has no byte after it, so it
+    // is fetched one byte early and shifted down.  my_state: byte offset of this lane's packed
+    // group in row row0 of the strip (the launch checks that the state is smaller than 2 GiB).
+    auto load_word = [&](uint32_t my_state, int i, int r) {
+        const uint32_t off = my_state + (uint32_t)(32 * (r / 4) + 4 * (r % 4) + i) * row_bytes;
+        const uint32_t is_last = off == last_group_off ? 1u : 0u;
+        uint32_t word;
+        __builtin_memcpy(&word, a.state + (off - is_last), 4);
+        return word >> (8 * is_last);
+    };
+
+    // Everything after a tile's hand-off: wait for the strip's decision, finish the rows of the
+    // strip, apply the ticks to the tile's columns.  False: the strip was not committed (the launch
+    // has failed) and nothing of it was written by this tile.
+    auto finish = [&](WideAcc& acc, int strip, int ct, float s_old, float v_old, int decision_naps)
+                      __attribute__((always_inline)) -> bool {
         const int m0 = strip * kWide, n0 = ct * kWide;
         StripControl* control = a.control + 2 * strip;
-        float* chain = a.chain + (size_t)strip * (2 * kWideChainSetFloats);
-
-        WideAcc acc;
-        wide_zero(acc);
-        wide_accumulate(a.grad_out + m0, a.x + n0, a.out_features, a.in_features, a.tokens, acc, lds, t);
-
-        // Old per-row values, read before anything of this strip is written: tile 0 overwrites
-        // them only after the strip has been committed, and commits happen after every tile of
-        // the strip has been here.
-        float s_old = 0.0f, v_old = 0.0f;
-        if (t.tid < kWide) {
-            s_old = a.scale[m0 + t.tid];
-            v_old = a.v[m0 + t.tid];
-        }
-        // byte offset of this lane's packed group in row row0 of the strip (the launch checks that
-        // the state is smaller than 2 GiB) and the element index of its first column there
-        const uint32_t my_state = (uint32_t)(m0 + row0) * row_bytes + 3u * (uint32_t)((n0 >> 2) + slot);
-        const uint32_t my_elem = (uint32_t)(m0 + row0) * (uint32_t)a.in_features +
-                                 (uint32_t)(n0 + 4 * slot + 2 * pair_half);
-        // One 4-byte load per lane and group; the tensor's last group has no byte after it, so it
-        // is fetched one byte early and shifted down.
-        auto load_word = [&](int i, int r) {
-            const uint32_t off = my_state + (uint32_t)(32 * (r / 4) + 4 * (r % 4) + i) * row_bytes;
-            const uint32_t is_last = off == last_group_off ? 1u : 0u;
-            uint32_t word;
-            __builtin_memcpy(&word, a.state + (off - is_last), 4);
-            return word >> (8 * is_last);
-        };
-
-        // ---- chain hand-off: step ct of all 64 chains of the strip's rows -------------------
-        if (!wait_for<false>(a, &control->published[0], ct, e.ok)) {
-            if (t.tid == 0) give_up(a, control);
-            return;
-        }
-#pragma unroll
-        for (int set = 0; set < (WITH_GS ? 2 : 1); ++set) {
-            float* my_chain = chain + set * kWideChainSetFloats + slot;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float in[16];
-#pragma unroll
-                for (int r = 0; r < 16; ++r) in[r] = ct > 0 ? load_shared_f32(my_chain + row_of(i, r) * 64) : 0.0f;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float v0, v1;
-                    if (set == 0) {
-                        v0 = acc[i][0][r] * acc[i][0][r];
-                        v1 = acc[i][1][r] * acc[i][1][r];
-                    } else {
-                        // g * t (kernels/compact_counter.cl:81-82): t from the element's code
-                        const uint32_t word = load_word(i, r) >> (12 * pair_half);
-                        v0 = acc[i][0][r] * (float)(code_q(word & 0x3fu, a.cd) - 1);
-                        v1 = acc[i][1][r] * (float)(code_q((word >> 6) & 0x3fu, a.cd) - 1);
-                    }
-                    const float first = (in[r] + v0) + v1;          // elements 0 and 1: the even lane's
-                    const float second = (from_even_lane(first) + v0) + v1;  // then 2 and 3: the odd lane's
-                    if (pair_half) store_shared_f32(my_chain + row_of(i, r) * 64, second);
-                }
-            }
-        }
-        stores_done();
-        __syncthreads();
-        if (t.tid == 0) {
-            __hip_atomic_store(&control->published[0], ct + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            // the last tile of the sequence commits the strip
-            if (ct + 1 == a.tiles_per_strip) {
-                __builtin_amdgcn_s_waitcnt(0);
-                cas_relaxed(&control->decision, 0, 1);
-            }
-        }
-
-        // ---- wait for the strip's decision ---------------------------------------------
-        bool committed = wait_for<true>(a, &control->decision, 0, e.ok);
+        const float* chain = a.chain + (size_t)strip * (2 * kWideChainSetFloats);
+        bool committed = wait_for<true>(a, &control->decision, 0, e.ok, decision_naps);
         if (t.tid == 0) {
             int d = committed ? load_relaxed(&control->decision) : give_up(a, control);
             if (d < 0 && committed) give_up(a, control);  // aborted by another tile: count this launch as failed
@@ -612,7 +554,7 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
         __syncthreads();
         committed = e.ok != 0;
         __syncthreads();
-        if (!committed) return;
+        if (!committed) return false;
 
         // ---- row statistics: every tile finishes the rows of its strip itself ---------------
         {
@@ -654,12 +596,15 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
         tc.lim_pos = (float)a.geom.lim_pos;
         tc.two_m24 = 1.0f / 16777216.0f;
         tc.seed_mix = seed_mix(a.seed);
+        const uint32_t my_state = (uint32_t)(m0 + row0) * row_bytes + 3u * (uint32_t)((n0 >> 2) + slot);
+        const uint32_t my_elem = (uint32_t)(m0 + row0) * (uint32_t)a.in_features +
+                                 (uint32_t)(n0 + 4 * slot + 2 * pair_half);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             // all 16 state loads are issued before the first tick
             uint32_t word[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) word[r] = load_word(i, r);
+            for (int r = 0; r < 16; ++r) word[r] = load_word(my_state, i, r);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = row_of(i, r);
@@ -685,7 +630,126 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
             }
         }
         __syncthreads();  // the row constants are rewritten by the next tile
+        return true;
+    };
+
+    // A tile whose strip ends in a later pass of the grid cannot be finished now without idling for
+    // the length of a pass: after its hand-off its accumulators go to one of the workgroup's two
+    // slots (two, because the next tile may have to be parked before this one can be finished)
+    // and the workgroup takes its next tile.  A parked tile is finished after the next tile has
+    // been dealt with -- by then the rest of its strip, which runs in that same pass, has published
+    // -- or, when there is no next tile, at the end.
+    float* my_slots = a.park ? a.park + (size_t)2 * ((int)blockIdx.x - a.park_first_wg) * kParkSlotFloats : nullptr;
+    int parked_strip = -1, parked_ct = 0, parked_slot = 0, next_slot = 0;
+    auto finish_parked = [&](int decision_naps) __attribute__((always_inline)) {
+        float* p = my_slots + (size_t)parked_slot * kParkSlotFloats;
+        WideAcc acc;
+#pragma unroll
+        for (int q = 0; q < 128; ++q) acc[q / 32][(q / 16) % 2][q % 16] = p[q * kWideThreads + t.tid];
+        float s_old = 0.0f, v_old = 0.0f;
+        if (t.tid < kWide) {
+            s_old = p[kWide * kWide + t.tid];
+            v_old = p[kWide * kWide + kWide + t.tid];
+        }
+        const bool ok = finish(acc, parked_strip, parked_ct, s_old, v_old, decision_naps);
+        parked_strip = -1;
+        return ok;
+    };
+
+    bool alive = true;
+    for (int tile = blockIdx.x; alive && tile < a.total_tiles; tile += gridDim.x) {
+        // once a workgroup has given up nothing new is started: a strip whose tiles have not all
+        // published cannot have been committed, and this tile has not published yet
+        if (t.tid == 0) e.ok = load_relaxed(a.status) == 0 ? 1 : 0;
+        __syncthreads();
+        const bool healthy = e.ok != 0;
+        __syncthreads();
+        if (!healthy) break;
+        const int strip = tile / a.tiles_per_strip;
+        const int ct = tile - strip * a.tiles_per_strip;
+        const int m0 = strip * kWide, n0 = ct * kWide;
+        StripControl* control = a.control + 2 * strip;
+        float* chain = a.chain + (size_t)strip * (2 * kWideChainSetFloats);
+
+        WideAcc acc;
+        wide_zero(acc);
+        wide_accumulate(a.grad_out + m0, a.x + n0, a.out_features, a.in_features, a.tokens, acc, lds, t);
+
+        // Old per-row values, read before anything of this strip is written: tile 0 overwrites
+        // them only after the strip has been committed, and commits happen after every tile of
+        // the strip has been here.
+        float s_old = 0.0f, v_old = 0.0f;
+        if (t.tid < kWide) {
+            s_old = a.scale[m0 + t.tid];
+            v_old = a.v[m0 + t.tid];
+        }
+        const uint32_t my_state = (uint32_t)(m0 + row0) * row_bytes + 3u * (uint32_t)((n0 >> 2) + slot);
+
+        // ---- chain hand-off: step ct of all 64 chains of the strip's rows -------------------
+        if (!wait_for<false>(a, &control->published[0], ct, e.ok)) {
+            if (t.tid == 0) give_up(a, control);
+            break;
+        }
+#pragma unroll
+        for (int set = 0; set < (WITH_GS ? 2 : 1); ++set) {
+            float* my_chain = chain + set * kWideChainSetFloats + slot;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float in[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) in[r] = ct > 0 ? load_shared_f32(my_chain + row_of(i, r) * 64) : 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float v0, v1;
+                    if (set == 0) {
+                        v0 = acc[i][0][r] * acc[i][0][r];
+                        v1 = acc[i][1][r] * acc[i][1][r];
+                    } else {
+                        // g * t (kernels/compact_counter.cl:81-82): t from the element's code
+                        const uint32_t word = load_word(my_state, i, r) >> (12 * pair_half);
+                        v0 = acc[i][0][r] * (float)(code_q(word & 0x3fu, a.cd) - 1);
+                        v1 = acc[i][1][r] * (float)(code_q((word >> 6) & 0x3fu, a.cd) - 1);
+                    }
+                    const float first = (in[r] + v0) + v1;          // elements 0 and 1: the even lane's
+                    const float second = (from_even_lane(first) + v0) + v1;  // then 2 and 3: the odd lane's
+                    if (pair_half) store_shared_f32(my_chain + row_of(i, r) * 64, second);
+                }
+            }
+        }
+        stores_done();
+        __syncthreads();
+        if (t.tid == 0) {
+            __hip_atomic_store(&control->published[0], ct + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the last tile of the sequence commits the strip
+            if (ct + 1 == a.tiles_per_strip) {
+                __builtin_amdgcn_s_waitcnt(0);
+                cas_relaxed(&control->decision, 0, 1);
+            }
+        }
+
+        const int pass = tile / (int)gridDim.x;
+        const int strip_last_pass = (strip * a.tiles_per_strip + a.tiles_per_strip - 1) / (int)gridDim.x;
+        if (my_slots && strip_last_pass > pass && (int)blockIdx.x >= a.park_first_wg) {
+            float* p = my_slots + (size_t)next_slot * kParkSlotFloats;
+#pragma unroll
+            for (int q = 0; q < 128; ++q) p[q * kWideThreads + t.tid] = acc[q / 32][(q / 16) % 2][q % 16];
+            if (t.tid < kWide) {
+                p[kWide * kWide + t.tid] = s_old;
+                p[kWide * kWide + kWide + t.tid] = v_old;
+            }
+            // the tile parked before this one: its strip ended in this pass
+            if (parked_strip >= 0) alive = finish_parked(0);
+            parked_strip = strip;
+            parked_ct = ct;
+            parked_slot = next_slot;
+            next_slot ^= 1;
+            continue;
+        }
+        alive = finish(acc, strip, ct, s_old, v_old, 0);
+        if (parked_strip >= 0) alive = finish_parked(0) && alive;
     }
+    // the rest of a parked tile's strip may still be a whole tile's time away: poll slowly
+    if (parked_strip >= 0) finish_parked(8);
 }
 
 __global__ void strip_clear_kernel(int* words, int n) {
@@ -741,7 +805,13 @@ static std::atomic<unsigned> g_spin_limit{kDefaultSpinLimit};
 // Which tiles a strip launch uses: 0 the wide ones where they keep the device busy, 1 the wide ones
 // whenever the shape allows them, 2 never (tests compare the two kernels).
 static std::atomic<int> g_wide_mode{0};
-void set_fused_strip_wide_mode(int mode) { g_wide_mode.store(mode >= 0 && mode <= 2 ? mode : 0); }
+// Test aid: the wide kernel's grid is held to this many workgroups (0: what the device holds), so
+// that small layers run in several passes and park tiles.
+static std::atomic<int> g_wide_grid_cap{0};
+void set_fused_strip_wide_mode(int mode, int grid_cap) {
+    g_wide_mode.store(mode >= 0 && mode <= 2 ? mode : 0);
+    g_wide_grid_cap.store(grid_cap > 0 ? grid_cap : 0);
+}
 
 unsigned fused_strip_spin_limit() { return g_spin_limit.load(); }
 void set_fused_strip_spin_limit(unsigned spins) { g_spin_limit.store(spins ? spins : kDefaultSpinLimit); }
@@ -751,10 +821,25 @@ bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch)
            out_features % kTile == 0 && in_features <= (size_t(1) << 31) / out_features;  // 32-bit element offsets
 }
 
-size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch) {
-    if (!fused_strip_supports(in_features, out_features, batch)) return 0;
+// Slots for parked tiles of the wide kernel: layers of more than 256 wide tiles -- more than one
+// pass of the persistent grid on a 256-CU device, so that strips can straddle passes -- get two
+// slots for each of the tiles_per_strip - 1 workgroups that may park (1 MiB per 4 slots).
+static size_t park_bytes(size_t in_features, size_t out_features, size_t batch) {
+    if (in_features % kWide || out_features % kWide || batch < (size_t)kBK || batch % kBK) return 0;
+    const size_t tiles_x = in_features / kWide, tiles = tiles_x * (out_features / kWide);
+    const int cap = g_wide_grid_cap.load();
+    if (tiles <= (size_t)(cap ? cap : 256) || tiles_x < 2) return 0;
+    return 2 * (tiles_x - 1) * (size_t)kParkSlotFloats * sizeof(float);
+}
+
+static size_t strip_base_bytes(size_t out_features) {
     const size_t strips = out_features / kTile;
     return kHeaderBytes + control_bytes(strips) + strips * kStripChainFloats * sizeof(float);
+}
+
+size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch) {
+    if (!fused_strip_supports(in_features, out_features, batch)) return 0;
+    return strip_base_bytes(out_features) + park_bytes(in_features, out_features, batch);
 }
 
 hipError_t fused_strip_take_failures(int* count) {
@@ -784,6 +869,8 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     a.status = reinterpret_cast<int*>(ws);
     a.control = reinterpret_cast<StripControl*>(ws + kHeaderBytes);
     a.chain = reinterpret_cast<float*>(ws + kHeaderBytes + control_bytes((size_t)strips));
+    a.park = nullptr;
+    a.park_first_wg = 0;
     a.tokens = tokens;
     a.in_features = in_features;
     a.out_features = out_features;
@@ -838,39 +925,53 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     if (err != hipSuccess) return err;
 
     // Wide tiles: whole 256 x 256 tiles, whole slabs, aligned operands -- and, unless forced, a shape
-    // whose strips come in rounds that keep at least four fifths of the CUs busy (4096 x 4096 is
-    // one round of 16 strips of 16 tiles, 11008 x 4096 three rounds for 2.69; 4096 x 11008 has 43
-    // tiles per strip, five strips per round and four rounds for 2.69, and stays on small tiles).
+    // whose tiles come in rounds that keep at least four fifths of the CUs busy.  With slots for
+    // parked tiles in the workspace a round is any 256 tiles (4096 x 11008: 688 tiles, three
+    // rounds for 2.69); without them a round is whole strips (4096 x 4096 is one round of 16 strips
+    // of 16 tiles; 4096 x 11008 would be four rounds of five strips of 43 tiles).
     const int wide_mode = g_wide_mode.load();
+    bool parking = false;
     if (wide_mode != 2 && vec_a && in_features % kWide == 0 && out_features % kWide == 0 && tokens >= kBK &&
         tokens % kBK == 0) {
         StripKernel wide = gs ? fused_strip_wide_kernel<true> : fused_strip_wide_kernel<false>;
         int wide_per_cu = 0;
         err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&wide_per_cu, wide, kWideThreads, 0);
         if (err != hipSuccess) return err;
-        const long capacity = (long)cus * wide_per_cu;
-        const long tiles_x = in_features / kWide, wide_strips = out_features / kWide;
+        const int cap = g_wide_grid_cap.load();
+        const long capacity = cap && cap < (long)cus * wide_per_cu ? cap : (long)cus * wide_per_cu;
+        const long tiles_x = in_features / kWide, wide_strips = out_features / kWide, tiles = tiles_x * wide_strips;
         if (capacity >= tiles_x) {
-            const long per_round = capacity / tiles_x;
-            const long rounds = (wide_strips + per_round - 1) / per_round;
-            if (wide_mode == 1 || wide_strips * tiles_x * 5 >= rounds * capacity * 4) {
+            parking = park_bytes((size_t)in_features, (size_t)out_features, (size_t)tokens) != 0 && tiles > capacity;
+            const long per_round = parking ? capacity : capacity / tiles_x * tiles_x;
+            const long rounds = (tiles + per_round - 1) / per_round;
+            if (wide_mode == 1 || tiles * 5 >= rounds * capacity * 4) {
                 kernel = wide;
                 threads = kWideThreads;
                 a.tiles_per_strip = (int)tiles_x;
-                a.total_tiles = (int)(wide_strips * tiles_x);
+                a.total_tiles = (int)tiles;
+            } else {
+                parking = false;
             }
         }
     }
 
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0);
     if (err != hipSuccess) return err;
-    const long capacity = (long)cus * per_cu;
+    long capacity = (long)cus * per_cu;
+    if (threads == kWideThreads && g_wide_grid_cap.load() && g_wide_grid_cap.load() < capacity)
+        capacity = g_wide_grid_cap.load();
     a.layer_wgs = cus;
     if (capacity < a.tiles_per_strip) return hipErrorLaunchOutOfResources;
     // a whole number of strips per pass of the persistent grid: a strip that straddled two passes
     // would park its early tiles' workgroups for the length of a pass
-    const long whole = capacity / a.tiles_per_strip * a.tiles_per_strip;
+    const long whole = parking ? capacity : capacity / a.tiles_per_strip * a.tiles_per_strip;
     const int grid = (int)(whole < a.total_tiles ? whole : a.total_tiles);
+    if (parking) {
+        // a tile is parked when its strip ends in a later pass: such tiles are the last ones of a
+        // pass and fewer than a strip has, so they sit on the last tiles_per_strip - 1 workgroups
+        a.park = reinterpret_cast<float*>(ws + strip_base_bytes((size_t)out_features));
+        a.park_first_wg = grid - (a.tiles_per_strip - 1);
+    }
 
     const int clear_words = (int)((kHeaderBytes + control_bytes((size_t)strips)) / sizeof(int));
     hipLaunchKernelGGL(strip_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, stream,

@@ -101,7 +101,9 @@ int mcc_fill_counter_state_u8(void* stream, uint8_t* dst, size_t n_groups, uint3
 
 void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins) { mcc::set_fused_strip_spin_limit(spins); }
 
-void mcc_compact_counter_fused_strip_set_tile_mode(int mode) { mcc::set_fused_strip_wide_mode(mode); }
+void mcc_compact_counter_fused_strip_set_tile_mode(int mode, int grid_cap) {
+    mcc::set_fused_strip_wide_mode(mode, grid_cap);
+}
 
 void mcc_contraction_spans_set_test_mode(unsigned polls, int start_first) {
     mcc::set_gemm_tn_wide_spans_test_mode(polls, start_first);

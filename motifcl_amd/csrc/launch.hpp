@@ -107,7 +107,9 @@ unsigned fused_strip_spin_limit();
 void set_fused_strip_spin_limit(unsigned spins);
 // Tiles of the strip step: 0 chosen by shape (256 x 256 where their rounds keep the device busy,
 // else 128 x 128), 1 wide whenever the shape allows, 2 never wide.  The result is the same bytes.
-void set_fused_strip_wide_mode(int mode);
+// grid_cap > 0 (a test aid) holds the wide kernel's grid to that many workgroups; it also enters
+// fused_strip_workspace_nbytes, which sizes the slots for parked tiles.
+void set_fused_strip_wide_mode(int mode, int grid_cap);
 // *busy: another strip launch of this process is still running on a different stream of the GPU
 // (nothing was enqueued).  Strip launches that give up a wait raise a per-device count that
 // fused_strip_take_failures reads and clears (the stream must have been synchronised).

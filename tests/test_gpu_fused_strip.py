@@ -49,11 +49,12 @@ def run_both(ops, n, n_in, n_out, C, seed, lr=HP["lr"], lr_scale=HP["lr_scale"])
 
 @pytest.fixture()
 def tile_mode():
-    """Selects the strip step's tiles: 0 by shape, 1 the 256 x 256 tiles wherever possible, 2 never."""
+    """Selects the strip step's tiles: 0 by shape, 1 the 256 x 256 tiles wherever possible, 2 never;
+    grid_cap holds the 256 x 256 kernel to that many workgroups."""
     import motifcl_amd
     L = motifcl_amd.load()
-    yield L.mcc_compact_counter_fused_strip_set_tile_mode
-    L.mcc_compact_counter_fused_strip_set_tile_mode(0)
+    yield lambda mode, grid_cap=0: L.mcc_compact_counter_fused_strip_set_tile_mode(mode, grid_cap)
+    L.mcc_compact_counter_fused_strip_set_tile_mode(0, 0)
 
 
 # (N, in, out, C): sides that are multiples of 256 and whole 16-token slabs, which the wide tiles take
@@ -78,6 +79,33 @@ def test_wide_strip_tiles_match_small_tiles_and_two_kernel_path(ops, tile_mode, 
     state, scale, v, _, _, (full, small) = run_both(ops, n, n_in, n_out, C, seed=n_in + n_out, lr_scale=lr_scale)
     tile_mode(1)
     _, _, _, _, _, (_, wide) = run_both(ops, n, n_in, n_out, C, seed=n_in + n_out, lr_scale=lr_scale)
+    assert not np.array_equal(full[0], state)
+    for a, b, c in zip(wide, small, full):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+        assert np.array_equal(a.view(np.uint8), c.view(np.uint8))
+
+
+# (N, in, out, C, workgroups): the grid held so small that strips straddle its passes
+PARKING_CASES = [
+    (48, 2048, 2048, 11, 44),   # 8 tiles a strip: four tiles parked in pass 0 by workgroups without a second tile
+    (48, 2048, 2048, 11, 12),   # ... parked tiles finished after the owner's next tile, several times
+    (32, 2048, 2048, 3, 10),    # workgroups 8 and 9 park in two passes running
+    (32, 1280, 1536, 11, 7),    # 5 tiles a strip, 30 tiles in passes of 7
+    (32, 11008, 768, 11, 50),   # 43 tiles a strip: 43 + 7 parked, ...
+]
+
+
+@pytest.mark.parametrize("lr_scale", [0.0, 0.05])
+@pytest.mark.parametrize("case", PARKING_CASES, ids=lambda s: "N%d_in%d_out%d_C%d_wgs%d" % s)
+def test_wide_strip_tiles_parked_between_passes(ops, tile_mode, case, lr_scale):
+    n, n_in, n_out, C, wgs = case
+    print("parking case", case, lr_scale, flush=True)
+    tile_mode(2)
+    plain = ops.fused_strip_workspace_nbytes(n_in, n_out, n)
+    state, scale, v, _, _, (full, small) = run_both(ops, n, n_in, n_out, C, seed=n_in + wgs, lr_scale=lr_scale)
+    tile_mode(1, wgs)
+    assert ops.fused_strip_workspace_nbytes(n_in, n_out, n) > plain   # slots for the parked tiles
+    _, _, _, _, _, (_, wide) = run_both(ops, n, n_in, n_out, C, seed=n_in + wgs, lr_scale=lr_scale)
     assert not np.array_equal(full[0], state)
     for a, b, c in zip(wide, small, full):
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
