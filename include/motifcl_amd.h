@@ -100,8 +100,10 @@ size_t mcc_compact_counter_fused_workspace_nbytes(size_t in_features, size_t out
  * runs without a buffer of the size of the weight gradient, or 0 when the shape
  * has no way smaller than the full workspace (tiny layers).  Layers whose in and
  * out are multiples of 128 with in >= 768 take the accumulator-resident strip
- * path: 512 bytes of partial row sums per output row plus a few control words
- * (5.6 MB for the largest layer of a 7B model instead of 180 MB).  Every other shape
+ * path: 512 bytes of partial row sums per output row plus a few control words,
+ * and, for layers of more than 256 tiles of 256 x 256, room to park 2 (in/256 - 1)
+ * such tiles between the passes of the kernel's grid (24 MB for the largest layer
+ * of a 7B model instead of 180 MB).  Every other shape
  * is updated band by band of an eighth of its output rows: the workspace holds
  * one band's gradient.  No counterpart in the reference, whose fused kernels
  * recompute the gradient instead of holding it.
@@ -112,8 +114,8 @@ size_t mcc_compact_counter_fused_strip_workspace_nbytes(size_t in_features, size
 /*
  * Waits for `stream` and reports whether every strip-path step of this process
  * on the current GPU since the last call completed: MCC_OK, or MCC_E_RUNTIME
- * when a step gave up a wait between tiles.  Such a step leaves whole 128-row
- * strips of its tensor without their update -- state, scale and v of those rows
+ * when a step gave up a wait between tiles.  Such a step leaves whole strips
+ * (128 or 256 rows) of its tensor without their update -- state, scale and v of those rows
  * are untouched, no strip is half-updated -- and the report clears the count.
  * The count lives in the library, per GPU, so it survives other layers' steps
  * through the same workspace; the workspace and shape arguments are not looked

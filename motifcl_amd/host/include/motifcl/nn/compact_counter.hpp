@@ -13,15 +13,15 @@ namespace motifcl::nn {
 
 // How the fused update holds the weight gradient while it needs the whole row's RMS:
 //   Full   contraction into f32[out,in] workspace slices, then the update kernel: the fastest way
-//          (about 10 percent on large layers; on small ones the only way to keep the GPU busy,
+//          (about 10 percent on a 7B-sized layer; on small ones the only way to keep the GPU busy,
 //          their token range being split over many workgroups).  The default.
 //   Small  no weight-sized buffer exists at any time, as in the reference
 //          (tests/test_memory_truth_gate.cpp:109-113).  Layers of 128-multiples with rows of at
 //          least 768 weights keep the gradient in the contraction's registers and exchange 512
-//          bytes of partial row sums per output row between the tiles of a 128-row strip; every
+//          bytes of partial row sums per output row between the tiles of a strip of 128 or 256 rows; every
 //          other layer is updated band by band of an eighth of its rows through a workspace of that
 //          size.  Any lr_scale.  check_fused_update() reports a strip step that gave up an
-//          inter-tile wait (such a step leaves whole 128-row strips without their update).
+//          inter-tile wait (such a step leaves whole strips without their update).
 // Small and Full give identical bytes wherever neither splits the tokens into chunks (fewer than
 // 512 tokens, or at least 1024 tiles of 128 x 128); elsewhere they add chunk sums in different
 // order and differ by that rounding, both within the tolerance the contraction is held to.
