@@ -279,13 +279,14 @@ def test_two_strip_updates_in_a_row_are_deterministic(ops):
         assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("wide", [False, True], ids=["tiles128", "tiles256"])
+@pytest.mark.parametrize("wide", [0, 1, 20], ids=["tiles128", "tiles256", "tiles256_parked"])
 def test_given_up_wait_is_reported_and_leaves_whole_strips_untouched(ops, tile_mode, wide):
     # a spin budget of one poll makes waits fail from the host side; the kernel must still drain,
     # the failure must surface through fused_check -- also after another layer has used the same
     # workspace -- and every strip (128 or 256 rows) must be either fully updated or untouched
     import motifcl_amd
-    tile_mode(1 if wide else 2)
+    # wide == 20: the 32 wide tiles run on 20 workgroups, four tiles of the second strip are parked
+    tile_mode(1 if wide else 2, wide if wide > 1 else 0)
     strip_rows = 256 if wide else 128
     from motifcl_amd.lib import MccError
     L = motifcl_amd.load()
