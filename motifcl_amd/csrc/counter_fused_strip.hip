@@ -505,6 +505,33 @@ __device__ __forceinline__ uint32_t pair_or(uint32_t x) {
 // the strip's 256 rows.  Only the workgroup that wrote a slot reads it, every thread its own values.
 constexpr int kParkSlotFloats = kWide * kWide + 2 * kWide;
 
+// The thread's coordinates recomputed from an index the compiler cannot see through: what the
+// epilogue derives from them (row offsets, state addresses) is then computed where it is used
+// instead of being hoisted over the tile loop and kept alive -- spilled -- across the contraction.
+struct WideEpiloguePos {
+    WideLane t;
+    int pair_half;  // 0: elements 0, 1 of the packed group; 1: elements 2, 3
+    int slot;       // the group's place in the tile = its chain
+    int row0;       // accumulator (i, j, r) is row row0 + 32 (r / 4) + 4 (r % 4) + i,
+                    // column 4 slot + 2 pair_half + j of the tile
+};
+__device__ __forceinline__ WideEpiloguePos fresh_wide_pos() {
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    WideEpiloguePos p;
+    p.t.tid = tid;
+    p.t.lane = tid & 63;
+    p.t.wave = tid >> 6;
+    p.t.l32 = p.t.lane & 31;
+    p.t.half = p.t.lane >> 5;
+    p.t.wm0 = (p.t.wave >> 2) * 128;
+    p.t.wn0 = (p.t.wave & 3) * 64;
+    p.pair_half = p.t.l32 & 1;
+    p.slot = (p.t.wn0 >> 2) + (p.t.l32 >> 1);
+    p.row0 = p.t.wm0 + 16 * p.t.half;
+    return p;
+}
+
 template <bool WITH_GS>
 MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
     __shared__ __attribute__((aligned(1024))) float lds[kWideBuffers * kWideSlabFloats];
@@ -520,10 +547,16 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
     const int groups_per_row = a.in_features >> 2;
     const uint32_t last_group_off = 3u * ((uint32_t)a.out_features * (uint32_t)groups_per_row - 1u);
     const uint32_t row_bytes = 3u * (uint32_t)groups_per_row;
-    const int pair_half = t.l32 & 1;                       // 0: elements 0, 1 of the packed group; 1: elements 2, 3
-    const int slot = (t.wn0 >> 2) + (t.l32 >> 1);          // the group's place in the tile = its chain
-    // accumulator (i, j, r) is row row0 + 32 (r / 4) + 4 (r % 4) + i, column 4 slot + 2 pair_half + j of the tile
-    const int row0 = t.wm0 + 16 * t.half;
+    // the epilogue's view of the thread, taken afresh at the start of each of its phases
+    WideLane te = t;
+    int pair_half = 0, slot = 0, row0 = 0;
+    auto refresh = [&]() __attribute__((always_inline)) {
+        const WideEpiloguePos p = fresh_wide_pos();
+        te = p.t;
+        pair_half = p.pair_half;
+        slot = p.slot;
+        row0 = p.row0;
+    };
     auto row_of = [&](int i, int r) { return row0 + 32 * (r / 4) + 4 * (r % 4) + i; };
 
     // One 4-byte load per lane and group; the tensor's last group has no byte after it, so it
@@ -542,11 +575,12 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
     // has failed) and nothing of it was written by this tile.
     auto finish = [&](WideAcc& acc, int strip, int ct, float s_old, float v_old, int decision_naps)
                       __attribute__((always_inline)) -> bool {
+        refresh();
         const int m0 = strip * kWide, n0 = ct * kWide;
         StripControl* control = a.control + 2 * strip;
         const float* chain = a.chain + (size_t)strip * (2 * kWideChainSetFloats);
         bool committed = wait_for<true>(a, &control->decision, 0, e.ok, decision_naps);
-        if (t.tid == 0) {
+        if (te.tid == 0) {
             int d = committed ? load_relaxed(&control->decision) : give_up(a, control);
             if (d < 0 && committed) give_up(a, control);  // aborted by another tile: count this launch as failed
             e.ok = d > 0 ? 1 : 0;
@@ -562,28 +596,28 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
             constexpr int kRowsPerWave = kWide / 8;
 #pragma unroll
             for (int set = 0; set < (WITH_GS ? 2 : 1); ++set) {
-                const float* mine = chain + set * kWideChainSetFloats + t.lane;
+                const float* mine = chain + set * kWideChainSetFloats + te.lane;
                 float part[kRowsPerWave];
 #pragma unroll
                 for (int rr = 0; rr < kRowsPerWave; ++rr)
-                    part[rr] = load_shared_f32(mine + (t.wave * kRowsPerWave + rr) * 64);
+                    part[rr] = load_shared_f32(mine + (te.wave * kRowsPerWave + rr) * 64);
 #pragma unroll
                 for (int rr = 0; rr < kRowsPerWave; ++rr) {
-                    const float sum = tree_sum(part[rr], t.lane);
-                    if (t.lane == 0) (set == 0 ? e.dn : e.k)[t.wave * kRowsPerWave + rr] = sum;  // parked; replaced below
+                    const float sum = tree_sum(part[rr], te.lane);
+                    if (te.lane == 0) (set == 0 ? e.dn : e.k)[te.wave * kRowsPerWave + rr] = sum;  // parked; replaced below
                 }
             }
         }
         __syncthreads();
-        if (t.tid < kWide) {
-            const RowStats rs = finish_row_stats(e.dn[t.tid], WITH_GS ? e.k[t.tid] : 0.0f, v_old, s_old, a.in_features,
+        if (te.tid < kWide) {
+            const RowStats rs = finish_row_stats(e.dn[te.tid], WITH_GS ? e.k[te.tid] : 0.0f, v_old, s_old, a.in_features,
                                                  WITH_GS ? a.lr_scale : 0.0f, a.rms_beta, a.rms_eps);
-            e.dn[t.tid] = rs.denom;
-            e.k[t.tid] = a.cd.Cf / rs.scale_new;
-            e.ratio[t.tid] = s_old / rs.scale_new;
+            e.dn[te.tid] = rs.denom;
+            e.k[te.tid] = a.cd.Cf / rs.scale_new;
+            e.ratio[te.tid] = s_old / rs.scale_new;
             if (ct == 0) {
-                a.v[m0 + t.tid] = rs.v_new;
-                a.scale[m0 + t.tid] = rs.scale_new;
+                a.v[m0 + te.tid] = rs.v_new;
+                a.scale[m0 + te.tid] = rs.scale_new;
             }
         }
         __syncthreads();
@@ -642,14 +676,15 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
     float* my_slots = a.park ? a.park + (size_t)2 * ((int)blockIdx.x - a.park_first_wg) * kParkSlotFloats : nullptr;
     int parked_strip = -1, parked_ct = 0, parked_slot = 0, next_slot = 0;
     auto finish_parked = [&](int decision_naps) __attribute__((always_inline)) {
+        refresh();
         float* p = my_slots + (size_t)parked_slot * kParkSlotFloats;
         WideAcc acc;
 #pragma unroll
-        for (int q = 0; q < 128; ++q) acc[q / 32][(q / 16) % 2][q % 16] = p[q * kWideThreads + t.tid];
+        for (int q = 0; q < 128; ++q) acc[q / 32][(q / 16) % 2][q % 16] = p[q * kWideThreads + te.tid];
         float s_old = 0.0f, v_old = 0.0f;
-        if (t.tid < kWide) {
-            s_old = p[kWide * kWide + t.tid];
-            v_old = p[kWide * kWide + kWide + t.tid];
+        if (te.tid < kWide) {
+            s_old = p[kWide * kWide + te.tid];
+            v_old = p[kWide * kWide + kWide + te.tid];
         }
         const bool ok = finish(acc, parked_strip, parked_ct, s_old, v_old, decision_naps);
         parked_strip = -1;
@@ -660,7 +695,7 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
     for (int tile = blockIdx.x; alive && tile < a.total_tiles; tile += gridDim.x) {
         // once a workgroup has given up nothing new is started: a strip whose tiles have not all
         // published cannot have been committed, and this tile has not published yet
-        if (t.tid == 0) e.ok = load_relaxed(a.status) == 0 ? 1 : 0;
+        if (te.tid == 0) e.ok = load_relaxed(a.status) == 0 ? 1 : 0;
         __syncthreads();
         const bool healthy = e.ok != 0;
         __syncthreads();
@@ -674,20 +709,21 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
         WideAcc acc;
         wide_zero(acc);
         wide_accumulate(a.grad_out + m0, a.x + n0, a.out_features, a.in_features, a.tokens, acc, lds, t);
+        refresh();
 
         // Old per-row values, read before anything of this strip is written: tile 0 overwrites
         // them only after the strip has been committed, and commits happen after every tile of
         // the strip has been here.
         float s_old = 0.0f, v_old = 0.0f;
-        if (t.tid < kWide) {
-            s_old = a.scale[m0 + t.tid];
-            v_old = a.v[m0 + t.tid];
+        if (te.tid < kWide) {
+            s_old = a.scale[m0 + te.tid];
+            v_old = a.v[m0 + te.tid];
         }
         const uint32_t my_state = (uint32_t)(m0 + row0) * row_bytes + 3u * (uint32_t)((n0 >> 2) + slot);
 
         // ---- chain hand-off: step ct of all 64 chains of the strip's rows -------------------
         if (!wait_for<false>(a, &control->published[0], ct, e.ok)) {
-            if (t.tid == 0) give_up(a, control);
+            if (te.tid == 0) give_up(a, control);
             break;
         }
 #pragma unroll
@@ -718,7 +754,7 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
         }
         stores_done();
         __syncthreads();
-        if (t.tid == 0) {
+        if (te.tid == 0) {
             __hip_atomic_store(&control->published[0], ct + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             // the last tile of the sequence commits the strip
             if (ct + 1 == a.tiles_per_strip) {
@@ -732,10 +768,10 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
         if (my_slots && strip_last_pass > pass && (int)blockIdx.x >= a.park_first_wg) {
             float* p = my_slots + (size_t)next_slot * kParkSlotFloats;
 #pragma unroll
-            for (int q = 0; q < 128; ++q) p[q * kWideThreads + t.tid] = acc[q / 32][(q / 16) % 2][q % 16];
-            if (t.tid < kWide) {
-                p[kWide * kWide + t.tid] = s_old;
-                p[kWide * kWide + kWide + t.tid] = v_old;
+            for (int q = 0; q < 128; ++q) p[q * kWideThreads + te.tid] = acc[q / 32][(q / 16) % 2][q % 16];
+            if (te.tid < kWide) {
+                p[kWide * kWide + te.tid] = s_old;
+                p[kWide * kWide + kWide + te.tid] = v_old;
             }
             // the tile parked before this one: its strip ended in this pass
             if (parked_strip >= 0) alive = finish_parked(0);
