@@ -184,6 +184,9 @@ __device__ __forceinline__ void wide_accumulate(const float* __restrict__ a, con
     // w + 8 of each, lane l the floats 4 l .. 4 l + 3 of the row
     const float* a_next = a + (size_t)t.wave * M + 4 * t.lane;
     const float* b_next = b + (size_t)t.wave * N + 4 * t.lane;
+    // the waits below count this call's copies: nothing older may be in flight (loads and stores
+    // share the counter and are not ordered against each other)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     for (int s = 0; s < kWideBuffers - 1 && s < slabs; ++s) {
         float* dst = lds + s * kWideSlabFloats + t.wave * kWide;
         __builtin_amdgcn_global_load_lds((global_ptr)a_next, (lds_ptr)dst, 16, 0, 0);
