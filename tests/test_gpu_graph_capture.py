@@ -25,9 +25,15 @@ def fresh(shape, seed):
     return state, scale, v, x, dy
 
 
+SMALL = [(256, 512, 256, 11), (320, 256, 384, 11)]   # the first splits its token range
+# 256 x 256 tiles: one round of them, then 688 tiles -- equal spans with hand-off words on the full
+# workspace, three passes with parked tiles on the strip workspace
+LARGE = [(32, 4096, 4096, 11), (32, 11008, 4096, 11)]
+
+
+@pytest.mark.parametrize("shapes", [SMALL, LARGE], ids=["small", "large"])
 @pytest.mark.parametrize("path", ["workspace", "strip"])
-def test_captured_steps_replay_like_eager(ops, path):
-    shapes = [(256, 512, 256, 11), (320, 256, 384, 11)]   # the first splits its token range
+def test_captured_steps_replay_like_eager(ops, path, shapes):
     if path == "strip":
         nbytes = [ops.fused_strip_workspace_nbytes(s[1], s[2], s[0]) for s in shapes]
     else:
