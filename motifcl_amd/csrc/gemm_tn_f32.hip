@@ -180,6 +180,15 @@ static bool wide_tiles_fill_the_device(int m, int n) {
     return tiles >= 256 && tiles * 100 >= rounds * 256 * 97;
 }
 
+// A smaller matrix whose token range the plan cuts into chunks: the wide tiles times the chunks
+// should come close to whole rounds (2048 x 768 at 16384 tokens: 24 tiles x 10 chunks = 240).
+static bool wide_chunks_fill_the_device(int m, int n, int splits) {
+    if (m % 256 || n % 256 || splits < 2) return false;
+    const long wgs = (long)(m / 256) * (n / 256) * splits;
+    const long rounds = (wgs + 255) / 256;
+    return wgs * 100 >= rounds * 256 * 85;
+}
+
 // For a matrix of `lines` x `across` wide tiles that is more than one round but not whole rounds:
 // how many lines make whole rounds of 256 tiles (0: none do).  11008 x 4096 is 43 x 16 tiles:
 // 32 lines are two rounds, the other 11 lines go to the small tiles.
@@ -251,7 +260,7 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
     const int wide_cols = wide_ok && plan.splits == 1 && wide_rows == 0 ? wide_block(n / 256, m / 256) : 0;
     if (mode == 1 && gemm_tn_bf16x6_supports(a, b, k, m, n, plan)) {
         e = launch_gemm_tn_bf16x6(stream, a, b, out, k, m, n, plan);
-    } else if (wide_ok && wide_tiles_fill_the_device(m, n)) {
+    } else if (wide_ok && (wide_tiles_fill_the_device(m, n) || wide_chunks_fill_the_device(m, n, plan.splits))) {
         e = launch_gemm_tn_wide(stream, a, b, out, k, m, n, n / 256, m / 256, plan.chunk, plan.splits);
     } else if (wide_ok && plan.splits == 1 && sync_words && gemm_tn_wide_spans_apply(k, m, n)) {
         e = launch_gemm_tn_wide_spans(stream, a, b, out, k, m, n, sync_words);
@@ -303,8 +312,12 @@ hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_
             const bool vec = j.m % 4 == 0 && j.n % 4 == 0 && (reinterpret_cast<uintptr_t>(j.a) & 15u) == 0 &&
                              (reinterpret_cast<uintptr_t>(j.b) & 15u) == 0;
             const long tiles = (long)((j.m + plan.tile - 1) / plan.tile) * ((j.n + plan.tile - 1) / plan.tile);
-            // a tensor of 1024 workgroups or more gains nothing from sharing a launch
+            // a tensor of 1024 workgroups or more gains nothing from sharing a launch, and one whose
+            // chunks fill the device with wide tiles is faster on those
             if (plan.tile != tile || !vec || tiles * plan.splits >= 1024) continue;
+            if (plan.tile == 128 && gemm_tn_wide_supports(j.a, j.b, j.k, j.m, j.n, plan.chunk) &&
+                wide_chunks_fill_the_device(j.m, j.n, plan.splits))
+                continue;
             if (g.n == kMaxGemmGroup || wgs > (1 << 30)) {
                 const hipError_t e = flush();
                 if (e != hipSuccess) return e;
