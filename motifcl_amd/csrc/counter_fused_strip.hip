@@ -423,7 +423,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void fused_strip_kernel(StripArgs 
         kq = tp.l32 & 3;
         // ---- ticks straight from the accumulators -----------------------------------------
         TickConsts tc;
-        tc.r = 0.0f;
+        tc.rd = 0.0;
         tc.neg_lr = -a.lr;
         tc.neg_lim_neg = -(float)a.geom.lim_neg;
         tc.lim_pos = (float)a.geom.lim_pos;
@@ -624,7 +624,7 @@ MCC_WIDE_KERNEL void fused_strip_wide_kernel(StripArgs a) {
 
         // ---- ticks straight from the accumulators -----------------------------------------
         TickConsts tc;
-        tc.r = 0.0f;
+        tc.rd = 0.0;
         tc.neg_lr = -a.lr;
         tc.neg_lim_neg = -(float)a.geom.lim_neg;
         tc.lim_pos = (float)a.geom.lim_pos;

@@ -73,7 +73,8 @@ MCC_HD uint32_t code_of(uint32_t word, int k) { return (word >> (6 * k)) & 0x3fu
 // ternary value).  (code * magic) >> 16 == code / lv for every code < 64.
 struct Codec {
     int C, lv;
-    uint32_t magic;
+    uint32_t magic;    // (code * magic) >> 16 == code / lv for code < 64
+    uint32_t c_magic;  // (n * c_magic) >> 16 == n / C for n < 5000 (C <= 11)
     float Cf, inv_c;
 };
 
@@ -82,6 +83,7 @@ MCC_HD Codec make_codec(int C) {
     cd.C = C;
     cd.lv = 2 * C - 1;
     cd.magic = 65536u / (uint32_t)cd.lv + 1u;
+    cd.c_magic = 65536u / (uint32_t)C + 1u;
     cd.Cf = (float)C;
     cd.inv_c = 1.0f / (float)C;
     return cd;
@@ -111,6 +113,7 @@ struct LutGeom {
     int lim_neg;   // clamp of floor(val) below, as a positive number
     int lim_pos;   // clamp of floor(val) above
     int width;     // number of distinct totals: lim_neg + lim_pos + 2
+    uint32_t width_magic;  // (idx * width_magic) >> 20 == idx / width for idx < rows * width
 };
 
 constexpr int kLutFinMaxBytes = 4480;  // C = 1: 64 rows x width 70
@@ -121,6 +124,7 @@ MCC_HD LutGeom lut_geom(const Codec& cd) {
     g.lim_neg = g.rows * cd.C + 1;
     g.lim_pos = 3 * cd.C;
     g.width = g.lim_neg + g.lim_pos + 2;
+    g.width_magic = (1u << 20) / (uint32_t)g.width + 1u;
     return g;
 }
 
@@ -128,7 +132,8 @@ MCC_HD LutGeom lut_geom(const Codec& cd) {
 MCC_HD uint32_t fin_entry(int total, int q, const Codec& cd) {
     const int C = cd.C;
     const int mag = total < 0 ? -total : total;
-    const int carry = total < 0 ? -(mag / C) : mag / C;  // trunc(ccv / Cf)
+    const int mq = (int)(((uint32_t)mag * cd.c_magic) >> 16);  // mag / C (mag <= rows * C + 2)
+    const int carry = total < 0 ? -mq : mq;               // trunc(ccv / Cf)
     int rem = total - carry * C;                          // ccv - carry * Cf
     const int nt = (q - 1) + carry;
     const int ct = nt < -1 ? -1 : (nt > 1 ? 1 : nt);
@@ -158,21 +163,25 @@ MCC_HD float c_reb_entry(uint32_t code, const Codec& cd, float ratio) {
 MCC_HD int fin_size(const LutGeom& g) { return g.rows * g.width; }
 
 MCC_HD void fill_fin_entry(int idx, const Codec& cd, const LutGeom& g, uint8_t* fin) {
-    const int q = idx / g.width;
+    const int q = (int)(((uint32_t)idx * g.width_magic) >> 20);  // idx / width
     const int til = idx - q * g.width;
     fin[idx] = (uint8_t)fin_entry(til - g.lim_neg, q, cd);
 }
 
-// Division by the per-row denominator, gw / dn, without a per-element reciprocal: with
-// r = RN(1/dn) computed once per row,
-//     q0 = RN(gw * r);  t = fma(-dn, q0, gw);  q1 = fma(t, r, q0);
-//     t  = fma(-dn, q1, gw);  q = fma(t, r, q1)
-// returns RN(gw / dn) exactly (Markstein: a faithful quotient corrected with the exact fma
-// residual and the correctly rounded reciprocal is the correctly rounded quotient), provided
-// no intermediate leaves the normal range.  That holds when dn is in [2^-40, 2^40] and every
-// gw of the row is zero or has |gw| in [2^-60, 2^50].  The row statistics pass collects what
-// the test needs: the sum of squares bounds |gw| from above, and the minimum over the row of
-// range_key(gw) bounds the non-zero |gw| from below.  Rows that fail take the plain division.
+// Division by the per-row denominator, gw / dn, without a per-element division: with
+// rd = RN64(1 / (double)dn) computed once per row,
+//     q = RN32(RN64((double)gw * rd))
+// is RN32(gw / dn) whenever that quotient is a normal binary32 number or zero.  Proof sketch: the
+// double product is q* (1 + e) with q* = gw / dn and |e| < 2^-51.9.  A rounding boundary of
+// binary32 next to q* is an odd multiple m of 2^(k-24) for q* in [2^k, 2^(k+1)); with the
+// significands G, D of gw and dn (integers below 2^24), |q* - m| = 2^(k-24) |G 2^s - M D| / D with
+// s in {24, 25} and M odd, and G 2^s = M D is impossible (D would need 24 factors of two), so
+// |q* - m| > 2^(k-48), sixteen times the error of the double product: both round to the same
+// binary32 number.  For subnormal quotients exact ties exist and the argument fails, so the row
+// statistics pass collects what bounds the quotients: dn in [2^-40, 2^40], the sum of squares
+// (|gw| from above) and the minimum over the row of range_key(gw) (non-zero |gw| from below,
+// 2^-60).  Rows that fail take the plain division.  Three instructions per element
+// (v_cvt_f64_f32, v_mul_f64, v_cvt_f32_f64) instead of a reciprocal product and four fmas.
 MCC_HD uint32_t float_bits(float f) {
 #if defined(__HIP_DEVICE_COMPILE__)
     return __float_as_uint(f);
@@ -201,15 +210,12 @@ MCC_HD int fast_division_from_min_abs(float dn, float row_sum_sq, float row_min_
 }
 
 template <bool FAST>
-MCC_HD float div_by_row(float gw, float dn, float r) {
+MCC_HD float div_by_row(float gw, float dn, double rd) {
     if (!FAST) return gw / dn;
-    float q = gw * r;
-    float t = fmaf(-dn, q, gw);
-    q = fmaf(t, r, q);
-    t = fmaf(-dn, q, gw);
-    q = fmaf(t, r, q);
-    return q;
+    return (float)((double)gw * rd);
 }
+
+MCC_HD double row_reciprocal(float dn) { return 1.0 / (double)dn; }
 
 MCC_HD float clamp_f(float x, float lo, float hi) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -221,7 +227,8 @@ MCC_HD float clamp_f(float x, float lo, float hi) {
 
 // Per-row constants of the tick (kernels/compact_counter.cl:118,123).
 struct TickConsts {
-    float dn, r;      // denom[row] and RN(1/denom[row])
+    float dn;         // denom[row]
+    double rd;        // row_reciprocal(denom[row])
     float k;          // Cf / s_new
     float neg_lr;     // -lr
     float neg_lim_neg, lim_pos;  // clamp of floor(val), as floats
@@ -238,7 +245,7 @@ struct TickConsts {
 template <bool FAST_DIV, typename CReb, typename QOff, typename Fin>
 MCC_HD uint32_t tick_code_from_product(uint32_t code, float gw, const TickConsts& tc, uint32_t first_product,
                                        CReb c_reb, QOff q_off, Fin fin) {
-    const float tick = (tc.neg_lr * div_by_row<FAST_DIV>(gw, tc.dn, tc.r)) * tc.k;
+    const float tick = (tc.neg_lr * div_by_row<FAST_DIV>(gw, tc.dn, tc.rd)) * tc.k;
     const float val = c_reb[code] + tick;
     const float f = floorf(val);
     const float frac = val - f;

@@ -15,12 +15,15 @@
 // 43 groups per lane for in = 11008) in VGPRs lets HBM see the gradient once:
 // 4 B (G) + 0.75 B (state read) + 0.75 B (state write) per weight.
 //
-// Why persistent waves over a batch: a wave alternates between waiting for its
-// row to arrive and ~45 VALU instructions per weight of tick arithmetic.  With
-// many more rows than resident waves the phases of different waves drift apart
-// and the memory system and the VALUs stay busy together; a single small
-// tensor is one synchronous round of load-then-compute.  The batched entry
-// point therefore walks the rows of up to 64 tensors in one launch.
+// Why one row per wave and no persistent grid: the workgroups of a launch are
+// dispatched in row order, so at any moment the rows in flight are a compact,
+// advancing window of the gradient and the state, and neighbouring rows --
+// whose bytes share DRAM pages -- are fetched at about the same time.  A
+// persistent grid striding over the rows loses that: its waves drift apart,
+// the window spreads over hundreds of megabytes, and the same loads and stores
+// run at 0.65 instead of 0.73 of the HBM peak (measured on the bare access
+// pattern; two rows per wave 0.72, four 0.68, eight 0.64).  The batched entry
+// point puts the tensor index on the grid's y axis.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -39,27 +42,38 @@ constexpr int kThreads = kWave;  // one wave per workgroup: the row index is a f
 struct BatchArgs {
     UpdateTensor t[kMaxUpdateBatch];
     int n_tensors;
-    int total_rows;
+    int total_rows;  // persistent kernels: rows of all tensors; dispatched kernels: unused
     Codec cd;
     LutGeom geom;
     float lr_scale, rms_beta, rms_eps;
 };
 static_assert(sizeof(BatchArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
-// Per-workgroup tables in LDS (see counter_math.hpp).  fin and q_off depend on C only and are
-// built once per launch; c_reb depends on the row's scale ratio and is rebuilt per row.
+// Per-workgroup tables in LDS (see counter_math.hpp).  All three depend on C only and are built
+// once per workgroup: c_f[code] is the residual counter as a float, and the rebased counter of
+// kernels/compact_counter.cl:124 is c_f[code] * (s_old / s_new) -- the product c_reb_entry forms.
 struct Luts {
     int q_off[64];   // first, so that the decode reads need no base-address add
-    float c_reb[64];
+    float c_f[64];   // 256 bytes behind q_off: one ds_read2st64_b32 fetches both
     uint8_t fin[kLutFinMaxBytes];
 };
 
 __device__ __forceinline__ void build_luts(Luts& l, const Codec& cd, const LutGeom& geom) {
-    for (int i = threadIdx.x; i < 64; i += blockDim.x) l.q_off[i] = q_off_entry((uint32_t)i, cd, geom);
+    for (int i = threadIdx.x; i < 64; i += blockDim.x) {
+        l.q_off[i] = q_off_entry((uint32_t)i, cd, geom);
+        l.c_f[i] = (float)code_c((uint32_t)i, cd);
+    }
     const int n = fin_size(geom);
     for (int i = threadIdx.x; i < n; i += blockDim.x) fill_fin_entry(i, cd, geom, l.fin);
     __syncthreads();
 }
+
+// c_reb[code] of the tick for a row whose scale changed: (float)c * (s_old / s_new).
+struct RebasedCounters {
+    const float* c_f;
+    float ratio;
+    __device__ __forceinline__ float operator[](uint32_t code) const { return c_f[code] * ratio; }
+};
 
 // A gradient element is read exactly once by the register-resident kernels: a non-temporal load
 // keeps it from displacing the state words (whose overlapping 4-byte loads do want the cache) and
@@ -166,15 +180,16 @@ __device__ __forceinline__ float wave_min_nonneg(float a, int lane) { return __u
 
 struct RowCtx {
     TickConsts tc;
+    float ratio;    // s_old / s_new: the rebase factor of the residual counters
     bool fast_div;  // wave-uniform
 };
 
-// Tree reduction, row epilogue, commit of v/scale, and the per-row c_reb table.  `exact_key()`
-// returns the lane's exact magnitude key over the row; it is called (by the whole wave) only when
-// the smallest magnitude cannot decide, i.e. when the row holds an exact zero.
+// Tree reduction, row epilogue and commit of v/scale.  `exact_key()` returns the lane's exact
+// magnitude key over the row; it is called (by the whole wave) only when the smallest magnitude
+// cannot decide, i.e. when the row holds an exact zero.
 template <bool WITH_GS, bool EXACT_KEY, typename KeyFn>
 __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTensor& t, int row, int lane,
-                                             const RowAcc& acc, Luts& l, KeyFn exact_key) {
+                                             const RowAcc& acc, KeyFn exact_key) {
     const float g_sq = tree_sum(acc.g_sq, lane);
     const float grad_s = WITH_GS ? tree_sum(acc.grad_s, lane) : 0.0f;
     const float s_old = t.scale[row];
@@ -193,12 +208,10 @@ __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTen
         t.v[row] = rs.v_new;
         t.scale[row] = rs.scale_new;  // commit (kernels/basic.cl:6-9); s_old stays in a register
     }
-    __syncthreads();  // the previous row's ticks have finished reading c_reb
-    l.c_reb[lane] = c_reb_entry((uint32_t)lane, a.cd, s_old / rs.scale_new);
-    __syncthreads();
     RowCtx rc;
+    rc.ratio = s_old / rs.scale_new;
     rc.tc.dn = rs.denom;
-    rc.tc.r = 1.0f / rs.denom;
+    rc.tc.rd = row_reciprocal(rs.denom);
     rc.tc.k = a.cd.Cf / rs.scale_new;
     rc.tc.neg_lr = -t.lr;
     rc.tc.neg_lim_neg = -(float)a.geom.lim_neg;
@@ -207,21 +220,21 @@ __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTen
     rc.tc.two_m24 = 1.0f / 16777216.0f;
     // two-register VOP2 forms issue faster than forms with a scalar or literal operand: keep the
     // per-row operands of the per-element instructions in vector registers
-    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24), "+v"(rc.tc.seed_mix));
+    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24), "+v"(rc.tc.seed_mix), "+v"(rc.tc.rd));
     rc.fast_div = __builtin_amdgcn_readfirstlane(fast > 0 ? 1 : 0) != 0;
     return rc;
 }
 
 __device__ __forceinline__ uint32_t no_exact_key() { return 0xffffffffu; }
 
-template <bool FAST_DIV>
-__device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], const TickConsts& tc,
+template <bool FAST_DIV, typename CReb>
+__device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], const TickConsts& tc, CReb c_reb,
                                                const Luts& l, uint32_t elem0) {
     uint32_t nw = 0;
     const uint32_t x0 = hash_first(elem0);  // elem0 is a multiple of 4: elements k share it up to ^k
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const uint32_t nc = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, x0 ^ (uint32_t)k, l.c_reb, l.q_off, l.fin);
+        const uint32_t nc = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, x0 ^ (uint32_t)k, c_reb, l.q_off, l.fin);
         nw |= nc << (6 * k);
     }
     return nw;
@@ -229,33 +242,35 @@ __device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], con
 
 // The same for a group whose first products come by addition (hash_delta): p0 is
 // hash_first(elem0) * kHashMul1 and d[k-1] the wave-uniform delta of element k.
-template <bool FAST_DIV>
-__device__ __forceinline__ uint32_t tick_group_deltas(uint32_t w, const float g[4], const TickConsts& tc,
+template <bool FAST_DIV, typename CReb>
+__device__ __forceinline__ uint32_t tick_group_deltas(uint32_t w, const float g[4], const TickConsts& tc, CReb c_reb,
                                                       const Luts& l, uint32_t p0, const uint32_t d[3]) {
     uint32_t nw = 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const uint32_t p = k == 0 ? p0 : p0 + d[k - 1];
-        const uint32_t nc = tick_code_from_product<FAST_DIV>(code_of(w, k), g[k], tc, p, l.c_reb, l.q_off, l.fin);
+        const uint32_t nc = tick_code_from_product<FAST_DIV>(code_of(w, k), g[k], tc, p, c_reb, l.q_off, l.fin);
         nw |= nc << (6 * k);
     }
     return nw;
 }
 
 // Tick pass over a row re-read from memory with byte-granular state access: the fallback for
-// rows of any length and alignment, and for rows that need the plain division.
-__device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, int lane, const TickConsts& tc,
+// rows of any length and alignment, for rows that need the plain division, and for rows whose
+// scale changes although lr_scale is zero (a scale outside its clamp range).
+__device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, int lane, const RowCtx& rc,
                                                const Luts& l, int group_begin = 0, int group_end = 0x7fffffff) {
     const int gpr = t.in_features >> 2;
     const int g_end = group_end < gpr ? group_end : gpr;
     const float* g_row = t.grad_w + (size_t)row * t.in_features;
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
     const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
+    const RebasedCounters c_reb{l.c_f, rc.ratio};
     for (int gi = group_begin + lane; gi < g_end; gi += kWave) {
         float g[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) g[k] = g_row[4 * gi + k];
-        const uint32_t nw = tick_group<false>(load_group(s_row + 3 * gi), g, tc, l, row_elem + 4u * (uint32_t)gi);
+        const uint32_t nw = tick_group<false>(load_group(s_row + 3 * gi), g, rc.tc, c_reb, l, row_elem + 4u * (uint32_t)gi);
         store_group(s_row + 3 * gi, nw);
     }
 }
@@ -288,19 +303,16 @@ __device__ __forceinline__ void load_row(const UpdateTensor& t, int row, int lan
     }
 }
 
-// One register-resident row: all loads are issued back to back (one contiguous burst per row,
-// which is also what the memory likes best: fetching the next row piecemeal during this row's
-// ticks was measured 10-30 % slower), then statistics, row epilogue and ticks.
+// One register-resident row whose loads have been issued (one contiguous burst per row): statistics,
+// row epilogue and ticks.  SCALED: the rebase factor multiplies the residual counters (lr_scale != 0).
 template <int ITERS, bool WITH_GS, bool EXACT>
 __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const UpdateTensor& t, int row, int lane,
-                                                    Luts& luts) {
+                                                    const Luts& luts, const float4 (&q)[ITERS],
+                                                    const uint32_t (&w)[ITERS]) {
     constexpr int kLast = ITERS - 1;
     const uint32_t gpr = (uint32_t)t.in_features >> 2;
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
     const bool last_live = EXACT || (uint32_t)lane + kWave * kLast < gpr;
-    float4 q[ITERS];
-    uint32_t w[ITERS];
-    load_row<ITERS, EXACT>(t, row, lane, q, w);
 
     RowAcc acc;
 #pragma unroll
@@ -310,7 +322,7 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
                             live ? q[j].w : 0.0f};
         accumulate<WITH_GS, false>(acc, g, live, w[j], a.cd);
     }
-    const RowCtx rc = finish_row<WITH_GS, false>(a, t, row, lane, acc, luts, [&]() {
+    const RowCtx rc = finish_row<WITH_GS, false>(a, t, row, lane, acc, [&]() {
         uint32_t key = 0xffffffffu;
 #pragma unroll
         for (int j = 0; j < ITERS; ++j) {
@@ -321,24 +333,41 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
         }
         return key;
     });
-    if (!rc.fast_div) {
-        apply_streamed(t, row, lane, rc.tc, luts);
+    // without lr_scale the scale only moves when it sits outside its clamp range
+    const bool unit_ratio = __builtin_amdgcn_readfirstlane(rc.ratio == 1.0f ? 1 : 0) != 0;
+    if (!rc.fast_div || (!WITH_GS && !unit_ratio)) {
+        apply_streamed(t, row, lane, rc, luts);
         return;
     }
+    const RebasedCounters rebased{luts.c_f, rc.ratio};
     const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
+    // EXACT rows: deltas of the first hash products, wave-uniform per 256-element span and the same
+    // for every span with equal bits 16..17 of the element index (a whole row, when it is short):
+    // they live in vector registers and are rewritten only when those bits change
+    uint32_t dv[3] = {0u, 0u, 0u};
+    uint32_t dv_bits = 4u;
 #pragma unroll
     for (int j = 0; j < ITERS; ++j) {
         const uint32_t gi = (uint32_t)lane + kWave * j;
         const float g[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
         uint32_t nw;
         if (EXACT) {
-            // wave-uniform: bits 16..17 of the element index are the same over this aligned span
             const uint32_t span = row_elem + 4u * kWave * j;
-            const uint32_t sbits = (span >> 16) & 3u;
-            const uint32_t d[3] = {hash_delta(sbits, 1), hash_delta(sbits, 2), hash_delta(sbits, 3)};
-            nw = tick_group_deltas<true>(w[j], g, rc.tc, luts, hash_first(span + 4u * (uint32_t)lane) * kHashMul1, d);
+            const uint32_t sbits = (span >> 16) & 3u;  // wave-uniform
+            if (sbits != dv_bits) {
+                dv_bits = sbits;
+                dv[0] = hash_delta(sbits, 1);
+                dv[1] = hash_delta(sbits, 2);
+                dv[2] = hash_delta(sbits, 3);
+                // opaque: the products stay products (x * M + d, not (x + d') * M)
+                asm volatile("" : "+v"(dv[0]), "+v"(dv[1]), "+v"(dv[2]));
+            }
+            const uint32_t p0 = hash_first(span + 4u * (uint32_t)lane) * kHashMul1;
+            nw = WITH_GS ? tick_group_deltas<true>(w[j], g, rc.tc, rebased, luts, p0, dv)
+                         : tick_group_deltas<true>(w[j], g, rc.tc, luts.c_f, luts, p0, dv);
         } else {
-            nw = tick_group<true>(w[j], g, rc.tc, luts, row_elem + 4u * gi);
+            nw = WITH_GS ? tick_group<true>(w[j], g, rc.tc, rebased, luts, row_elem + 4u * gi)
+                         : tick_group<true>(w[j], g, rc.tc, luts.c_f, luts, row_elem + 4u * gi);
         }
         if (j < kLast || last_live) store_group(s_row + 3u * gi, nw);
     }
@@ -347,7 +376,7 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
 // One row of any length and alignment: read twice (the second read hits L2).
 template <bool WITH_GS>
 __device__ __forceinline__ void update_row_streamed(const BatchArgs& a, const UpdateTensor& t, int row,
-                                                    int lane, Luts& luts) {
+                                                    int lane, const Luts& luts) {
     const int gpr = t.in_features >> 2;
     const float* g_row = t.grad_w + (size_t)row * t.in_features;
     const uint8_t* s_row = t.state + (size_t)row * gpr * 3;
@@ -358,8 +387,8 @@ __device__ __forceinline__ void update_row_streamed(const BatchArgs& a, const Up
         for (int k = 0; k < 4; ++k) g[k] = g_row[4 * gi + k];
         accumulate<WITH_GS, true>(acc, g, true, load_group(s_row + 3 * gi), a.cd);
     }
-    const RowCtx rc = finish_row<WITH_GS, true>(a, t, row, lane, acc, luts, no_exact_key);
-    apply_streamed(t, row, lane, rc.tc, luts);
+    const RowCtx rc = finish_row<WITH_GS, true>(a, t, row, lane, acc, no_exact_key);
+    apply_streamed(t, row, lane, rc, luts);
 }
 
 // State word of group gc of a row; `last_row` (wave-uniform) tells that the row is the tensor's
@@ -380,7 +409,7 @@ constexpr int kChunk = 8;
 
 template <bool WITH_GS>
 __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const UpdateTensor& t, int row,
-                                                    int lane, Luts& luts) {
+                                                    int lane, const Luts& luts) {
     const uint32_t gpr = (uint32_t)t.in_features >> 2;
     const int iters = (int)((gpr + kWave - 1) / kWave);
     const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
@@ -406,11 +435,12 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
             accumulate<WITH_GS, true>(acc, g, live, WITH_GS ? w[j] : 0u, a.cd);
         }
     }
-    const RowCtx rc = finish_row<WITH_GS, true>(a, t, row, lane, acc, luts, no_exact_key);
+    const RowCtx rc = finish_row<WITH_GS, true>(a, t, row, lane, acc, no_exact_key);
     if (!rc.fast_div) {
-        apply_streamed(t, row, lane, rc.tc, luts);
+        apply_streamed(t, row, lane, rc, luts);
         return;
     }
+    const RebasedCounters rebased{luts.c_f, rc.ratio};
     const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
     for (int c0 = 0; c0 < iters; c0 += kChunk) {
         float4 q[kChunk];
@@ -427,7 +457,7 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
             if (c0 + j < iters) {  // wave-uniform
                 const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(c0 + j);
                 const float g[4] = {q[j].x, q[j].y, q[j].z, q[j].w};
-                const uint32_t nw = tick_group<true>(w[j], g, rc.tc, luts, row_elem + 4u * gi);
+                const uint32_t nw = tick_group<true>(w[j], g, rc.tc, rebased, luts, row_elem + 4u * gi);
                 if (gi < gpr) store_group(s_row + 3u * gi, nw);
             }
         }
@@ -439,6 +469,29 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
 // rows and 2 for the longest.
 constexpr int min_waves(int iters) { return iters <= 10 ? 4 : (iters <= 16 ? 3 : 2); }
 
+// Waves (= rows) per workgroup of the dispatched kernels: the workgroup builds the tables once.
+constexpr int kRowsPerGroup = 4;
+
+// Register-resident rows, one per wave; blockIdx.y is the tensor, blockIdx.x * kRowsPerGroup the
+// workgroup's first row.  Every tensor of a launch has the same out_features.
+template <int ITERS, bool WITH_GS, bool EXACT>
+__global__ __launch_bounds__(kWave* kRowsPerGroup, min_waves(ITERS)) void update_rows_kernel(BatchArgs a) {
+    __shared__ Luts luts;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const UpdateTensor t = a.t[blockIdx.y];
+    const int row_v = blockIdx.x * kRowsPerGroup + wave;
+    const bool valid = row_v < t.out_features;  // wave-uniform
+    const int row = valid ? row_v : t.out_features - 1;
+    // the row's loads go out first; the tables are built while they are in flight
+    float4 q[ITERS];
+    uint32_t w[ITERS];
+    load_row<ITERS, EXACT>(t, row, lane, q, w);
+    build_luts(luts, a.cd, a.geom);
+    if (!valid) return;
+    update_row_resident<ITERS, WITH_GS, EXACT>(a, t, row, lane, luts, q, w);
+}
+
 // The tensor that holds row `grow` of the launch's concatenated row space; ti only moves forward.
 // Everything here depends on blockIdx and kernel arguments only, so it lives in scalar registers.
 __device__ __forceinline__ UpdateTensor locate_row(const BatchArgs& a, int grow, int& ti) {
@@ -448,20 +501,7 @@ __device__ __forceinline__ UpdateTensor locate_row(const BatchArgs& a, int grow,
     return a.t[ti];
 }
 
-template <int ITERS, bool WITH_GS, bool EXACT>
-__global__ __launch_bounds__(kThreads, min_waves(ITERS)) void update_rows_kernel(BatchArgs a) {
-    __shared__ Luts luts;
-    build_luts(luts, a.cd, a.geom);
-    const int lane = threadIdx.x;
-    int ti = 0;
-    for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
-        const int grow = __builtin_amdgcn_readfirstlane(grow_v);
-        const UpdateTensor t = locate_row(a, grow, ti);
-        update_row_resident<ITERS, WITH_GS, EXACT>(a, t, grow - t.row_start, lane, luts);
-    }
-}
-
-// Rows of any length and alignment, streamed (read twice).
+// Rows of any length and alignment, streamed (read twice); persistent one-wave workgroups.
 template <bool WITH_GS>
 __global__ __launch_bounds__(kThreads, 4) void update_rows_streamed_kernel(BatchArgs a) {
     __shared__ Luts luts;
@@ -489,19 +529,20 @@ __global__ __launch_bounds__(kThreads, 4) void update_rows_long_kernel(BatchArgs
 }
 
 // ---------------------------------------------------------------------------
-// Long rows: W cooperating waves per row.  Wave w keeps iterations [w*J, (w+1)*J) of the row in
-// its registers, so a row of up to 64*J*W groups is register-resident with J*5 instead of
-// ITERS*5 row registers per lane, and three or four waves per SIMD still fit.  The reference's
-// per-lane partial sums are sequential in the iteration index, so the running sums are handed
-// from wave to wave through LDS (W-1 barriers); the last wave owns the tree, the row epilogue
-// and the commit, and publishes the tick constants for everybody's share of the tick pass.
+// Long rows: W cooperating waves per row, one row per workgroup (blockIdx.x the row, blockIdx.y
+// the tensor).  Wave w keeps iterations [w*J, (w+1)*J) of the row in its registers, so a row of
+// up to 64*J*W groups is register-resident with J*5 instead of ITERS*5 row registers per lane,
+// and three or four waves per SIMD still fit.  The reference's per-lane partial sums are
+// sequential in the iteration index, so the running sums are handed from wave to wave through
+// LDS (W-1 barriers); the last wave owns the tree, the row epilogue and the commit, and
+// publishes the tick constants for everybody's share of the tick pass.
 // ---------------------------------------------------------------------------
 struct SplitShared {
     Luts luts;
     float part_sq[kWave];
     float part_gs[kWave];
     uint32_t part_key[kWave];
-    TickConsts tc;
+    RowCtx rc;
     int fast_div;
 };
 
@@ -510,129 +551,110 @@ constexpr int min_waves_split(int j) { return j <= 6 ? 4 : 3; }
 template <int J, int W, bool WITH_GS>
 __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_split_kernel(BatchArgs a) {
     __shared__ SplitShared sh;
-    build_luts(sh.luts, a.cd, a.geom);
     const int lane = threadIdx.x & (kWave - 1);
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    int ti = 0;
-    for (int grow_v = blockIdx.x; grow_v < a.total_rows; grow_v += gridDim.x) {
-        const int grow = __builtin_amdgcn_readfirstlane(grow_v);
-        const UpdateTensor t = locate_row(a, grow, ti);
-        const int row = grow - t.row_start;
-        const bool last_row = row == t.out_features - 1;
-        const uint32_t gpr = (uint32_t)t.in_features >> 2;
-        const int iters = (int)((gpr + kWave - 1) / kWave);
-        const int j0 = w * J;
-        const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
-        uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    const UpdateTensor t = a.t[blockIdx.y];
+    const int row = blockIdx.x;
+    const bool last_row = row == t.out_features - 1;
+    const uint32_t gpr = (uint32_t)t.in_features >> 2;
+    const int iters = (int)((gpr + kWave - 1) / kWave);
+    const int j0 = w * J;
+    const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
+    uint8_t* s_row = t.state + (size_t)row * gpr * 3;
 
-        float4 q[J];
-        uint32_t words[J];
+    float4 q[J];
+    uint32_t words[J];
+#pragma unroll
+    for (int jj = 0; jj < J; ++jj) {
+        const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
+        const uint32_t gc = gi < gpr ? gi : gpr - 1;
+        q[jj] = load_grad4_once(g_row + gc);
+        words[jj] = load_row_word(s_row, gc, gpr, last_row);
+    }
+    build_luts(sh.luts, a.cd, a.geom);  // while the row is in flight
+    // What does not depend on the order happens before the hand-off, in all waves at once: the
+    // squares, the products with t, and the minimum of the magnitude keys (a minimum may be
+    // taken in any order).  Only the additions travel wave 0 -> 1 -> ... -> W-1.  (Long
+    // per-wave stretches have no registers to spare for the squares and do it all in turn.)
+    constexpr bool kPre = J <= 11;
+    float sq[kPre ? J : 1][4], gt[kPre && WITH_GS ? J : 1][4];
+    uint32_t my_key = 0xffffffffu;
+    if (kPre) {
 #pragma unroll
         for (int jj = 0; jj < J; ++jj) {
-            const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
-            const uint32_t gc = gi < gpr ? gi : gpr - 1;
-            q[jj] = load_grad4_once(g_row + gc);
-            words[jj] = load_row_word(s_row, gc, gpr, last_row);
-        }
-        // What does not depend on the order happens before the hand-off, in all waves at once: the
-        // squares, the products with t, and the minimum of the magnitude keys (a minimum may be
-        // taken in any order).  Only the additions travel wave 0 -> 1 -> ... -> W-1.  (Long
-        // per-wave stretches have no registers to spare for the squares and do it all in turn.)
-        constexpr bool kPre = J <= 11;
-        float sq[kPre ? J : 1][4], gt[kPre && WITH_GS ? J : 1][4];
-        uint32_t my_key = 0xffffffffu;
-        if (kPre) {
+            const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+            const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
+                                live ? q[jj].w : 0.0f};
+            my_key = umin3(my_key, range_key(g[0]), range_key(g[1]));
+            my_key = umin3(my_key, range_key(g[2]), range_key(g[3]));
 #pragma unroll
-            for (int jj = 0; jj < J; ++jj) {
-                const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
-                const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
-                                    live ? q[jj].w : 0.0f};
-                my_key = umin3(my_key, range_key(g[0]), range_key(g[1]));
-                my_key = umin3(my_key, range_key(g[2]), range_key(g[3]));
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    sq[jj][k] = g[k] * g[k];
-                    if (WITH_GS) gt[jj][k] = g[k] * (float)(code_q(code_of(words[jj], k), a.cd) - 1);
-                }
+            for (int k = 0; k < 4; ++k) {
+                sq[jj][k] = g[k] * g[k];
+                if (WITH_GS) gt[jj][k] = g[k] * (float)(code_q(code_of(words[jj], k), a.cd) - 1);
             }
         }
-        RowAcc acc;
+    }
+    RowAcc acc;
 #pragma unroll
-        for (int step = 0; step < W; ++step) {
-            if (w == step) {
-                if (step > 0) {
-                    acc.g_sq = sh.part_sq[lane];
-                    acc.grad_s = sh.part_gs[lane];
-                    acc.min_key = sh.part_key[lane];
-                }
-                if (kPre) {
-                    acc.min_key = umin(acc.min_key, my_key);
+    for (int step = 0; step < W; ++step) {
+        if (w == step) {
+            if (step > 0) {
+                acc.g_sq = sh.part_sq[lane];
+                acc.grad_s = sh.part_gs[lane];
+                acc.min_key = sh.part_key[lane];
+            }
+            if (kPre) {
+                acc.min_key = umin(acc.min_key, my_key);
 #pragma unroll
-                    for (int jj = 0; jj < J; ++jj)
+                for (int jj = 0; jj < J; ++jj)
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            acc.g_sq = acc.g_sq + sq[jj][k];
-                            if (WITH_GS) acc.grad_s = acc.grad_s + gt[jj][k];
-                        }
-                } else {
-#pragma unroll
-                    for (int jj = 0; jj < J; ++jj) {
-                        const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
-                        const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
-                                            live ? q[jj].w : 0.0f};
-                        accumulate<WITH_GS, true>(acc, g, live, words[jj], a.cd);
+                    for (int k = 0; k < 4; ++k) {
+                        acc.g_sq = acc.g_sq + sq[jj][k];
+                        if (WITH_GS) acc.grad_s = acc.grad_s + gt[jj][k];
                     }
-                }
-                if (step < W - 1) {
-                    sh.part_sq[lane] = acc.g_sq;
-                    sh.part_gs[lane] = acc.grad_s;
-                    sh.part_key[lane] = acc.min_key;
-                }
-            }
-            __syncthreads();
-        }
-        if (w == W - 1) {
-            const float g_sq = tree_sum(acc.g_sq, lane);
-            const float grad_s = WITH_GS ? tree_sum(acc.grad_s, lane) : 0.0f;
-            const uint32_t min_key = wave_min(acc.min_key, lane);
-            const float s_old = t.scale[row];
-            const float v_old = t.v[row];
-            const RowStats rs = finish_row_stats(g_sq, grad_s, v_old, s_old, t.in_features, a.lr_scale,
-                                                 a.rms_beta, a.rms_eps);
-            sh.luts.c_reb[lane] = c_reb_entry((uint32_t)lane, a.cd, s_old / rs.scale_new);
-            if (lane == 0) {
-                t.v[row] = rs.v_new;
-                t.scale[row] = rs.scale_new;
-                TickConsts tc;
-                tc.dn = rs.denom;
-                tc.r = 1.0f / rs.denom;
-                tc.k = a.cd.Cf / rs.scale_new;
-                tc.neg_lr = -t.lr;
-                tc.neg_lim_neg = -(float)a.geom.lim_neg;
-                tc.lim_pos = (float)a.geom.lim_pos;
-                tc.seed_mix = seed_mix(t.seed);
-                tc.two_m24 = 1.0f / 16777216.0f;
-                sh.tc = tc;
-                sh.fast_div = row_takes_fast_division(rs.denom, g_sq, min_key) ? 1 : 0;
-            }
-        }
-        __syncthreads();
-        TickConsts tc = sh.tc;
-        asm volatile("" : "+v"(tc.neg_lr), "+v"(tc.k), "+v"(tc.two_m24));  // VGPR multipliers
-        const bool fast = __builtin_amdgcn_readfirstlane(sh.fast_div) != 0;
-        if (!fast) {
-            apply_streamed(t, row, lane, tc, sh.luts, j0 * kWave, (j0 + J) * kWave);
-            continue;
-        }
-        const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
+            } else {
 #pragma unroll
-        for (int jj = 0; jj < J; ++jj) {
-            if (j0 + jj < iters) {  // wave-uniform
-                const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
-                const float g[4] = {q[jj].x, q[jj].y, q[jj].z, q[jj].w};
-                const uint32_t nw = tick_group<true>(words[jj], g, tc, sh.luts, row_elem + 4u * gi);
-                if (gi < gpr) store_group(s_row + 3u * gi, nw);
+                for (int jj = 0; jj < J; ++jj) {
+                    const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+                    const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
+                                        live ? q[jj].w : 0.0f};
+                    accumulate<WITH_GS, true>(acc, g, live, words[jj], a.cd);
+                }
             }
+            if (step < W - 1) {
+                sh.part_sq[lane] = acc.g_sq;
+                sh.part_gs[lane] = acc.grad_s;
+                sh.part_key[lane] = acc.min_key;
+            }
+        }
+        if (step < W - 1) __syncthreads();
+    }
+    if (w == W - 1) {
+        const RowCtx rc = finish_row<WITH_GS, true>(a, t, row, lane, acc, no_exact_key);
+        if (lane == 0) {
+            sh.rc = rc;
+            sh.fast_div = rc.fast_div ? 1 : 0;
+        }
+    }
+    __syncthreads();
+    RowCtx rc = sh.rc;
+    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24), "+v"(rc.tc.seed_mix), "+v"(rc.tc.rd));  // VGPR operands
+    const bool fast = __builtin_amdgcn_readfirstlane(sh.fast_div) != 0;
+    const bool unit_ratio = __builtin_amdgcn_readfirstlane(rc.ratio == 1.0f ? 1 : 0) != 0;
+    if (!fast || (!WITH_GS && !unit_ratio)) {
+        apply_streamed(t, row, lane, rc, sh.luts, j0 * kWave, (j0 + J) * kWave);
+        return;
+    }
+    const RebasedCounters rebased{sh.luts.c_f, rc.ratio};
+    const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
+#pragma unroll
+    for (int jj = 0; jj < J; ++jj) {
+        if (j0 + jj < iters) {  // wave-uniform
+            const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
+            const float g[4] = {q[jj].x, q[jj].y, q[jj].z, q[jj].w};
+            const uint32_t nw = WITH_GS ? tick_group<true>(words[jj], g, rc.tc, rebased, sh.luts, row_elem + 4u * gi)
+                                        : tick_group<true>(words[jj], g, rc.tc, sh.luts.c_f, sh.luts, row_elem + 4u * gi);
+            if (gi < gpr) store_group(s_row + 3u * gi, nw);
         }
     }
 }
@@ -647,18 +669,11 @@ int device_cu_count() {
     return cus;
 }
 
+// Every tensor of `a` has the rows of a.t[0]: one workgroup per kRowsPerGroup rows and tensor.
 template <int ITERS, bool WITH_GS, bool EXACT>
 hipError_t launch_variant(hipStream_t stream, const BatchArgs& a) {
-    static int blocks_per_cu = [] {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_kernel<ITERS, WITH_GS, EXACT>, kThreads, 0) !=
-                hipSuccess || n <= 0)
-            n = 2;
-        return n;
-    }();
-    const int resident = device_cu_count() * blocks_per_cu;
-    const dim3 grid(a.total_rows < resident ? a.total_rows : resident);
-    hipLaunchKernelGGL((update_rows_kernel<ITERS, WITH_GS, EXACT>), grid, dim3(kThreads), 0, stream, a);
+    const dim3 grid((unsigned)((a.t[0].out_features + kRowsPerGroup - 1) / kRowsPerGroup), (unsigned)a.n_tensors);
+    hipLaunchKernelGGL((update_rows_kernel<ITERS, WITH_GS, EXACT>), grid, dim3(kWave * kRowsPerGroup), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -679,15 +694,7 @@ hipError_t launch_streamed_variant(hipStream_t stream, const BatchArgs& a) {
 
 template <int J, int W, bool WITH_GS>
 hipError_t launch_split_variant(hipStream_t stream, const BatchArgs& a) {
-    static int blocks_per_cu = [] {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, update_rows_split_kernel<J, W, WITH_GS>, kWave * W, 0) !=
-                hipSuccess || n <= 0)
-            n = 1;
-        return n;
-    }();
-    const int resident = device_cu_count() * blocks_per_cu;
-    const dim3 grid(a.total_rows < resident ? a.total_rows : resident);
+    const dim3 grid((unsigned)a.t[0].out_features, (unsigned)a.n_tensors);
     hipLaunchKernelGGL((update_rows_split_kernel<J, W, WITH_GS>), grid, dim3(kWave * W), 0, stream, a);
     return hipGetLastError();
 }
@@ -752,6 +759,10 @@ int iters_class(const UpdateTensor& t) {
     return 0;
 }
 
+// Dispatched classes put the tensor on the grid's y axis and need equal out_features per launch;
+// the persistent fallbacks walk one concatenated row space.
+bool class_is_dispatched(int cls) { return cls != 0 && cls != kLongClass; }
+
 hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
     switch (cls) {
 #define MCC_CASE(N)                                  \
@@ -770,8 +781,8 @@ hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
 }  // namespace
 
 // Enqueues the update-only step for `n` tensors (already validated).  Tensors are grouped by
-// the register-resident variant their row length needs; each group goes out in launches of at
-// most kMaxUpdateBatch tensors.
+// the kernel variant their row length needs (and, for the dispatched variants, by their row
+// count); each group goes out in launches of at most kMaxUpdateBatch tensors.
 hipError_t launch_update_batch(hipStream_t stream, const UpdateTensor* tensors, size_t n, int C,
                                float lr_scale, float rms_beta, float rms_eps) {
     BatchArgs a;
@@ -798,10 +809,12 @@ hipError_t launch_update_batch(hipStream_t stream, const UpdateTensor* tensors, 
     }
     for (size_t i = 0; i < n; ++i) {
         if (done[i]) continue;
+        const bool by_rows = class_is_dispatched(cls[i]);
         a.n_tensors = 0;
         a.total_rows = 0;
         for (size_t j = i; j < n; ++j) {
             if (done[j] || cls[j] != cls[i]) continue;
+            if (by_rows && tensors[j].out_features != tensors[i].out_features) continue;
             // total_rows stays below 2^31: flush before the row space of one launch gets there
             if (a.n_tensors == kMaxUpdateBatch || a.total_rows > (1 << 30) - tensors[j].out_features) {
                 const hipError_t e = launch_class(stream, cls[i], a);

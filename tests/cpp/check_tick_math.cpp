@@ -34,12 +34,17 @@ int main(int argc, char** argv) {
         std::vector<float> c_reb(64);
         for (uint32_t code = 0; code < 64; ++code) q_off[code] = mcc::q_off_entry(code, cd, g);
         for (int i = 0; i < mcc::fin_size(g); ++i) mcc::fill_fin_entry(i, cd, g, fin.data());
+        // the table build's divisions by C and by the table width
+        for (int n = 0; n < 5000; ++n)
+            if ((int)(((uint32_t)n * cd.c_magic) >> 16) != n / C) { std::printf("division by C fails C=%d n=%d\n", C, n); return 2; }
+        for (int i = 0; i < mcc::fin_size(g); ++i)
+            if ((int)(((uint32_t)i * g.width_magic) >> 20) != i / g.width) { std::printf("division by the width fails C=%d i=%d\n", C, i); return 2; }
         // (code * magic) >> 16 == code / lv
         for (uint32_t code = 0; code < 64; ++code)
             if (mcc::code_q(code, cd) != (int)code / cd.lv) { std::printf("magic division fails C=%d code=%u\n", C, code); return 2; }
         auto make_tc = [&](float dn, float s_old, float s_new, float lr, uint32_t seed) {
             mcc::TickConsts tc;
-            tc.dn = dn; tc.r = 1.0f / dn; tc.k = cd.Cf / s_new; tc.neg_lr = -lr;
+            tc.dn = dn; tc.rd = mcc::row_reciprocal(dn); tc.k = cd.Cf / s_new; tc.neg_lr = -lr;
             tc.neg_lim_neg = -(float)g.lim_neg; tc.lim_pos = (float)g.lim_pos;
             tc.seed_mix = mcc::seed_mix(seed); tc.two_m24 = 1.0f / 16777216.0f;
             for (uint32_t code = 0; code < 64; ++code) c_reb[code] = mcc::c_reb_entry(code, cd, s_old / s_new);
