@@ -17,6 +17,7 @@
 #else
 #define MCC_HD inline
 #endif
+#define MCC_HDC constexpr MCC_HD  // also usable in constant expressions (the tables are built at compile time)
 
 namespace mcc {
 
@@ -78,8 +79,8 @@ struct Codec {
     float Cf, inv_c;
 };
 
-MCC_HD Codec make_codec(int C) {
-    Codec cd;
+MCC_HDC Codec make_codec(int C) {
+    Codec cd{};
     cd.C = C;
     cd.lv = 2 * C - 1;
     cd.magic = 65536u / (uint32_t)cd.lv + 1u;
@@ -90,7 +91,7 @@ MCC_HD Codec make_codec(int C) {
 }
 
 // t + 1 = code / lv  (kernels/compact_counter.cl:10)
-MCC_HD int code_q(uint32_t code, const Codec& cd) { return (int)((code * cd.magic) >> 16); }
+MCC_HDC int code_q(uint32_t code, const Codec& cd) { return (int)((code * cd.magic) >> 16); }
 
 // ---------------------------------------------------------------------------
 // The tick after val = c_reb + tick is a function of three small integers:
@@ -118,8 +119,8 @@ struct LutGeom {
 
 constexpr int kLutFinMaxBytes = 4480;  // C = 1: 64 rows x width 70
 
-MCC_HD LutGeom lut_geom(const Codec& cd) {
-    LutGeom g;
+MCC_HDC LutGeom lut_geom(const Codec& cd) {
+    LutGeom g{};
     g.rows = 63 / cd.lv + 1;
     g.lim_neg = g.rows * cd.C + 1;
     g.lim_pos = 3 * cd.C;
@@ -129,7 +130,7 @@ MCC_HD LutGeom lut_geom(const Codec& cd) {
 }
 
 // New code for old q = t + 1 and integer total = ccv (kernels/compact_counter.cl:129-136).
-MCC_HD uint32_t fin_entry(int total, int q, const Codec& cd) {
+MCC_HDC uint32_t fin_entry(int total, int q, const Codec& cd) {
     const int C = cd.C;
     const int mag = total < 0 ? -total : total;
     const int mq = (int)(((uint32_t)mag * cd.c_magic) >> 16);  // mag / C (mag <= rows * C + 2)
@@ -148,11 +149,11 @@ MCC_HD uint32_t fin_entry(int total, int q, const Codec& cd) {
 // c_reb is the rebased residual counter of kernels/compact_counter.cl:124; it depends on the
 // row through the scale ratio only, so it is tabulated once per row (64 products) instead of
 // once per weight.
-MCC_HD int code_c(uint32_t code, const Codec& cd) {
+MCC_HDC int code_c(uint32_t code, const Codec& cd) {
     return (int)code - code_q(code, cd) * cd.lv - (cd.C - 1);
 }
 
-MCC_HD int q_off_entry(uint32_t code, const Codec& cd, const LutGeom& g) {
+MCC_HDC int q_off_entry(uint32_t code, const Codec& cd, const LutGeom& g) {
     return code_q(code, cd) * g.width + g.lim_neg;
 }
 
@@ -160,9 +161,9 @@ MCC_HD float c_reb_entry(uint32_t code, const Codec& cd, float ratio) {
     return (float)code_c(code, cd) * ratio;
 }
 
-MCC_HD int fin_size(const LutGeom& g) { return g.rows * g.width; }
+MCC_HDC int fin_size(const LutGeom& g) { return g.rows * g.width; }
 
-MCC_HD void fill_fin_entry(int idx, const Codec& cd, const LutGeom& g, uint8_t* fin) {
+MCC_HDC void fill_fin_entry(int idx, const Codec& cd, const LutGeom& g, uint8_t* fin) {
     const int q = (int)(((uint32_t)idx * g.width_magic) >> 20);  // idx / width
     const int til = idx - q * g.width;
     fin[idx] = (uint8_t)fin_entry(til - g.lim_neg, q, cd);
@@ -271,7 +272,9 @@ struct RowStats {
 MCC_HD RowStats finish_row_stats(float sum_sq, float sum_gt, float v_old, float scale_old,
                                  int in_features, float lr_scale, float rms_beta, float rms_eps) {
     const float gsq = sum_sq / (float)in_features;
-    const float gs = sum_gt / sqrtf((float)in_features);
+    // lr_scale == 0: the product below is +-0 for every finite gs and the scale stays as it is
+    // (up to its clamp), so the square root and the division are skipped
+    const float gs = lr_scale != 0.0f ? sum_gt / sqrtf((float)in_features) : 0.0f;
     const float a = rms_beta * v_old;
     const float b = (1.0f - rms_beta) * gsq;
     RowStats r;

@@ -49,22 +49,46 @@ struct BatchArgs {
 };
 static_assert(sizeof(BatchArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
-// Per-workgroup tables in LDS (see counter_math.hpp).  All three depend on C only and are built
-// once per workgroup: c_f[code] is the residual counter as a float, and the rebased counter of
-// kernels/compact_counter.cl:124 is c_f[code] * (s_old / s_new) -- the product c_reb_entry forms.
-struct Luts {
+// Per-workgroup tables in LDS (see counter_math.hpp).  All three depend on C only: c_f[code] is
+// the residual counter as a float, and the rebased counter of kernels/compact_counter.cl:124 is
+// c_f[code] * (s_old / s_new) -- the product c_reb_entry forms.  The tables of every valid C
+// (3 (2C - 1) <= 64, i.e. C <= 11) are built at compile time and sit in the code object; a
+// workgroup copies the ones of its C into LDS (16 bytes per thread) instead of computing them.
+struct alignas(16) Luts {
     int q_off[64];   // first, so that the decode reads need no base-address add
     float c_f[64];   // 256 bytes behind q_off: one ds_read2st64_b32 fetches both
     uint8_t fin[kLutFinMaxBytes];
 };
+static_assert(sizeof(Luts) % 16 == 0, "copied in 16-byte pieces");
+
+constexpr int kMaxC = 11;
+
+struct LutsByC {
+    Luts c[kMaxC];
+};
+
+constexpr LutsByC make_all_luts() {
+    LutsByC all{};
+    for (int C = 1; C <= kMaxC; ++C) {
+        Luts& l = all.c[C - 1];
+        const Codec cd = make_codec(C);
+        const LutGeom geom = lut_geom(cd);
+        for (int i = 0; i < 64; ++i) {
+            l.q_off[i] = q_off_entry((uint32_t)i, cd, geom);
+            l.c_f[i] = (float)code_c((uint32_t)i, cd);
+        }
+        for (int i = 0, n = fin_size(geom); i < n; ++i) fill_fin_entry(i, cd, geom, l.fin);
+    }
+    return all;
+}
+
+__device__ const LutsByC kLutsByC = make_all_luts();
 
 __device__ __forceinline__ void build_luts(Luts& l, const Codec& cd, const LutGeom& geom) {
-    for (int i = threadIdx.x; i < 64; i += blockDim.x) {
-        l.q_off[i] = q_off_entry((uint32_t)i, cd, geom);
-        l.c_f[i] = (float)code_c((uint32_t)i, cd);
-    }
-    const int n = fin_size(geom);
-    for (int i = threadIdx.x; i < n; i += blockDim.x) fill_fin_entry(i, cd, geom, l.fin);
+    const int pieces = (2 * 64 * 4 + fin_size(geom) + 15) / 16;
+    const uint4* src = reinterpret_cast<const uint4*>(&kLutsByC.c[cd.C - 1]);
+    uint4* dst = reinterpret_cast<uint4*>(&l);
+    for (int i = threadIdx.x; i < pieces; i += blockDim.x) dst[i] = src[i];
     __syncthreads();
 }
 
@@ -227,17 +251,24 @@ __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTen
 
 __device__ __forceinline__ uint32_t no_exact_key() { return 0xffffffffu; }
 
+// Four 6-bit codes -> the group's 24-bit word, as three shift-or instructions.
+__device__ __forceinline__ uint32_t pack_codes(const uint32_t nc[4]) {
+    uint32_t nw = nc[0];
+    asm("v_lshl_or_b32 %0, %1, 6, %0" : "+v"(nw) : "v"(nc[1]));
+    asm("v_lshl_or_b32 %0, %1, 12, %0" : "+v"(nw) : "v"(nc[2]));
+    asm("v_lshl_or_b32 %0, %1, 18, %0" : "+v"(nw) : "v"(nc[3]));
+    return nw;
+}
+
 template <bool FAST_DIV, typename CReb>
 __device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], const TickConsts& tc, CReb c_reb,
                                                const Luts& l, uint32_t elem0) {
-    uint32_t nw = 0;
+    uint32_t nc[4];
     const uint32_t x0 = hash_first(elem0);  // elem0 is a multiple of 4: elements k share it up to ^k
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const uint32_t nc = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, x0 ^ (uint32_t)k, c_reb, l.q_off, l.fin);
-        nw |= nc << (6 * k);
-    }
-    return nw;
+    for (int k = 0; k < 4; ++k)
+        nc[k] = tick_code<FAST_DIV>(code_of(w, k), g[k], tc, x0 ^ (uint32_t)k, c_reb, l.q_off, l.fin);
+    return pack_codes(nc);
 }
 
 // The same for a group whose first products come by addition (hash_delta): p0 is
@@ -245,14 +276,13 @@ __device__ __forceinline__ uint32_t tick_group(uint32_t w, const float g[4], con
 template <bool FAST_DIV, typename CReb>
 __device__ __forceinline__ uint32_t tick_group_deltas(uint32_t w, const float g[4], const TickConsts& tc, CReb c_reb,
                                                       const Luts& l, uint32_t p0, const uint32_t d[3]) {
-    uint32_t nw = 0;
+    uint32_t nc[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const uint32_t p = k == 0 ? p0 : p0 + d[k - 1];
-        const uint32_t nc = tick_code_from_product<FAST_DIV>(code_of(w, k), g[k], tc, p, c_reb, l.q_off, l.fin);
-        nw |= nc << (6 * k);
+        nc[k] = tick_code_from_product<FAST_DIV>(code_of(w, k), g[k], tc, p, c_reb, l.q_off, l.fin);
     }
-    return nw;
+    return pack_codes(nc);
 }
 
 // Tick pass over a row re-read from memory with byte-granular state access: the fallback for
