@@ -130,12 +130,33 @@ __device__ __forceinline__ uint32_t load_group_dword(const uint8_t* p) {
     return w;
 }
 
+// The forms the register-resident kernels use: every state byte is read once and written once per
+// step, and marking BOTH the load and the stores non-temporal lets the bare access pattern run at
+// 0.79 instead of 0.74 of the HBM peak (the hint on the loads alone costs 12 %, on the stores
+// alone nothing).
+typedef uint32_t __attribute__((aligned(1))) unaligned_u32;
+typedef uint16_t __attribute__((aligned(1))) unaligned_u16;
+
+__device__ __forceinline__ uint32_t load_group_dword_once(const uint8_t* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const unaligned_u32*>(p));
+}
+
+__device__ __forceinline__ void store_group_once(uint8_t* p, uint32_t w) {
+    __builtin_nontemporal_store((uint16_t)w, reinterpret_cast<unaligned_u16*>(p));
+    __builtin_nontemporal_store((uint8_t)(w >> 16), p + 2);
+}
+
 // The same for a group that may be the tensor's last (`tail`): that one has no byte after it, so
 // it is fetched one byte early and shifted down.  The tensor holds at least two groups (the
 // launch sends smaller ones to the byte-granular kernel), so the byte before exists.
 __device__ __forceinline__ uint32_t load_group_dword_or_tail(const uint8_t* p, bool tail) {
     const uint32_t back = tail ? 1u : 0u;
     return load_group_dword(p - back) >> (8u * back);
+}
+
+__device__ __forceinline__ uint32_t load_group_dword_or_tail_once(const uint8_t* p, bool tail) {
+    const uint32_t back = tail ? 1u : 0u;
+    return load_group_dword_once(p - back) >> (8u * back);
 }
 
 // Row statistics of one group (kernels/compact_counter.cl:78-83) plus what decides whether the
@@ -328,8 +349,8 @@ __device__ __forceinline__ void load_row(const UpdateTensor& t, int row, int lan
         const uint32_t gc = j < kLast ? (uint32_t)lane + kWave * j : gc_last;
         q[j] = load_grad4_once(g_row + gc);
         // only the row's last iteration can hold the tensor's last group
-        w[j] = j < kLast ? load_group_dword(s_row + 3u * gc)
-                         : load_group_dword_or_tail(s_row + 3u * gc, last_row && gc == gpr - 1);
+        w[j] = j < kLast ? load_group_dword_once(s_row + 3u * gc)
+                         : load_group_dword_or_tail_once(s_row + 3u * gc, last_row && gc == gpr - 1);
     }
 }
 
@@ -399,7 +420,7 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
             nw = WITH_GS ? tick_group<true>(w[j], g, rc.tc, rebased, luts, row_elem + 4u * gi)
                          : tick_group<true>(w[j], g, rc.tc, luts.c_f, luts, row_elem + 4u * gi);
         }
-        if (j < kLast || last_live) store_group(s_row + 3u * gi, nw);
+        if (j < kLast || last_live) store_group_once(s_row + 3u * gi, nw);
     }
 }
 
@@ -599,7 +620,8 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
         const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
         const uint32_t gc = gi < gpr ? gi : gpr - 1;
         q[jj] = load_grad4_once(g_row + gc);
-        words[jj] = load_row_word(s_row, gc, gpr, last_row);
+        words[jj] = last_row ? load_group_dword_or_tail_once(s_row + 3u * gc, gc == gpr - 1)
+                             : load_group_dword_once(s_row + 3u * gc);
     }
     build_luts(sh.luts, a.cd, a.geom);  // while the row is in flight
     // What does not depend on the order happens before the hand-off, in all waves at once: the
@@ -684,7 +706,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
             const float g[4] = {q[jj].x, q[jj].y, q[jj].z, q[jj].w};
             const uint32_t nw = WITH_GS ? tick_group<true>(words[jj], g, rc.tc, rebased, sh.luts, row_elem + 4u * gi)
                                         : tick_group<true>(words[jj], g, rc.tc, sh.luts.c_f, sh.luts, row_elem + 4u * gi);
-            if (gi < gpr) store_group(s_row + 3u * gi, nw);
+            if (gi < gpr) store_group_once(s_row + 3u * gi, nw);
         }
     }
 }
