@@ -144,12 +144,13 @@ int mcc_compact_counter_fused_check(void* stream, const void* workspace, size_t 
  *     property tests/test_memory_truth_gate.cpp:109-113 of the reference asks
  *     for.  Any lr_scale.  On the strip path (see the size query) the update is
  *     applied from the contraction's accumulators; x must be 16-byte aligned;
- *     tiles of one row strip wait for each other on the device, so a second
- *     such call issued on another stream while one is still running is refused
- *     with MCC_E_INVALID (order the two), every wait is bounded, and
- *     mcc_compact_counter_fused_check reports a wait that was given up.  On a
- *     stream under graph capture the refusal is not applied: do not replay two
- *     such graphs side by side.
+ *     tiles of one row strip wait for each other on the device, so two such
+ *     steps must not run side by side on one GPU: a call on another stream than
+ *     the previous strip call is ordered behind it on the device (the stream
+ *     waits for an event recorded after that call; the host does not wait),
+ *     every wait is bounded, and mcc_compact_counter_fused_check reports a
+ *     wait that was given up.  On a stream under graph capture no such order
+ *     is added: do not replay two such graphs side by side.
  * The ways produce identical bytes whenever none of them splits the tokens into
  * chunks, i.e. for fewer than 512 tokens or layers of at least 1024 tiles of
  * 128 x 128 (mcc_compact_counter_fused_workspace_nbytes == out*in*4); where
@@ -188,6 +189,12 @@ int mcc_compact_counter_apply_update_fused(
  *   - it fails with MCC_E_INVALID and a message that names both sizes.
  * All calls on one GPU share that GPU's array, which keeps the last call's
  * contents: two calls that overlap in time on one GPU (different streams) race.
+ * The first call on a GPU looks up the array's address there (and, for a shape
+ * on the strip path, creates the event that orders strip steps of different
+ * streams): make that first call outside graph capture; later calls may be
+ * captured and replayed.  A step that took the strip path reports a given-up
+ * wait through mcc_compact_counter_fused_check, like the lent-workspace call
+ * (its workspace arguments are not looked at: pass a null pointer and 0).
  * Arguments and validation are those of mcc_compact_counter_apply_update_fused
  * without the workspace.
  */
@@ -237,8 +244,9 @@ int mcc_compact_counter_apply_update_fused_batched(
 
 /*
  * How the weight-gradient contraction (inside the two-kernel fused step and in
- * mcc_matmul_transpose_a_f32) multiplies.  Process-wide; no counterpart in the
- * reference.
+ * mcc_matmul_transpose_a_f32) multiplies.  A setting of the calling thread: it
+ * governs the calls that thread makes afterwards and no other thread's.  No
+ * counterpart in the reference.
  *   MCC_CONTRACTION_FP32    the fp32 matrix instruction (default)
  *   MCC_CONTRACTION_BF16X6  both operands split into three bf16 terms, six bf16
  *                           matrix passes per product: per-product error of one

@@ -4,9 +4,12 @@
  * Nothing here has a counterpart in the reference and nothing here is part of
  * the drop-in boundary (that is motifcl_amd.h): a shader-clock probe used by
  * the benchmark to report the clock the kernels ran at, the generator of the
- * benchmark's synthetic inputs, and the knob that lets a test force the bounded
- * device-side wait of the strip-workspace fused step to give up.  Conventions (status codes, mcc_last_error) are those of
- * motifcl_amd.h.
+ * benchmark's synthetic inputs, and the knobs that let a test force the bounded
+ * device-side waits to give up or a small layer to take the paths of a large
+ * one.  Every knob is a setting of the calling thread: a thread that never
+ * touches them runs on the defaults whatever other threads set, and no entry
+ * point of motifcl_amd.h changes its answer because of them.  Conventions
+ * (status codes, mcc_last_error) are those of motifcl_amd.h.
  */
 #ifndef MOTIFCL_AMD_DIAG_H
 #define MOTIFCL_AMD_DIAG_H
@@ -32,10 +35,14 @@ void mcc_compact_counter_fused_strip_set_spin_limit(unsigned spins);
  * write the same bytes; tests use the switch to compare them on small shapes.
  * grid_cap > 0 holds the 256 x 256 kernel to that many workgroups, so that a
  * small layer runs in several passes of its persistent grid and parks tiles
- * whose strip ends in a later pass; the cap also enters the strip workspace
- * size (the slots for parked tiles), so set it before sizing the workspace.  0 restores the device's own capacity.
+ * whose strip ends in a later pass; such a step needs the workspace size
+ * mcc_compact_counter_fused_strip_workspace_nbytes_for_grid returns for that
+ * cap (the slots for parked tiles; the public size query never depends on the
+ * cap) and is rejected with a smaller one.  0 restores the device's own capacity.
  */
 void mcc_compact_counter_fused_strip_set_tile_mode(int mode, int grid_cap);
+size_t mcc_compact_counter_fused_strip_workspace_nbytes_for_grid(size_t in_features, size_t out_features,
+                                                                 size_t batch, int grid_cap);
 
 /*
  * The contraction of shapes that are more than two but not a whole number of rounds of

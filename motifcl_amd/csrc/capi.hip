@@ -47,7 +47,8 @@ constexpr size_t kIntMax = static_cast<size_t>(std::numeric_limits<int>::max());
 
 // 0: weight-gradient contraction on the fp32 matrix instruction; 1: split-bf16 form where the
 // shape allows it
-std::atomic<int> g_contraction_mode{0};
+// the calling thread's setting: other threads' calls are not affected and no call sees it change
+thread_local int g_contraction_mode = 0;
 
 // Shared shape/codec checks.  `what` names the operation in messages.
 bool check_codec(const char* what, size_t C, size_t in_features, size_t out_features) {
@@ -386,15 +387,10 @@ int mcc::fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* 
     hipError_t e;
     if (small && plan.kind == SmallPlan::kStrip) {
         ScopedKernelTimer timer("fused_strip", s);
-        bool busy = false;
         e = mcc::launch_fused_strip(s, state, scale, v, grad_out, x, workspace, (int)C, (int)in_features,
                                     (int)out_features, (int)batch, lr, lr_scale, rms_beta, rms_eps, seed,
-                                    mcc::fused_strip_spin_limit(), &busy);
+                                    mcc::fused_strip_spin_limit(), workspace_nbytes);
         if (e != hipSuccess) return hip_fail(e, "compact-counter fused strip update launch failed");
-        if (busy)
-            return fail(MCC_E_INVALID,
-                        "compact-counter fused update with the strip workspace: another such step is still running on a "
-                        "different stream of this GPU; order the two (one stream, or an event between them)");
         return MCC_OK;
     }
     if (small) {
@@ -424,7 +420,7 @@ int mcc::fused_update(void* stream, uint8_t* state, size_t state_nbytes, float* 
                               ? reinterpret_cast<int*>(grad_w + out_features * in_features)
                               : nullptr;
         e = mcc::launch_gemm_tn_f32(s, grad_out, x, grad_w, (int)batch, (int)out_features, (int)in_features, grad_w,
-                                    g_contraction_mode.load(), 0, nullptr, sync_words);
+                                    g_contraction_mode, 0, nullptr, sync_words);
     }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
     {
@@ -535,7 +531,7 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
     }
     // every tensor has been validated: nothing below fails for a reason the arguments could show
     // another contraction mode than the fp32 instruction: tensor by tensor, each in its own region
-    if (g_contraction_mode.load() != MCC_CONTRACTION_FP32) {
+    if (g_contraction_mode != MCC_CONTRACTION_FP32) {
         ws = static_cast<uint8_t*>(workspace);
         for (size_t i = 0; i < n_tensors; ++i) {
             const mcc_fused_tensor& t = tensors[i];
@@ -569,11 +565,11 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
 int mcc_set_contraction_mode(int mode) {
     if (mode != MCC_CONTRACTION_FP32 && mode != MCC_CONTRACTION_BF16X6)
         return fail(MCC_E_INVALID, "unknown contraction mode");
-    g_contraction_mode.store(mode);
+    g_contraction_mode = mode;
     return MCC_OK;
 }
 
-int mcc_get_contraction_mode(void) { return g_contraction_mode.load(); }
+int mcc_get_contraction_mode(void) { return g_contraction_mode; }
 
 int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, const float* b,
                                size_t b_nbytes, float* c, size_t c_nbytes, size_t k, size_t m,
@@ -608,7 +604,7 @@ int mcc_matmul_transpose_a_f32(void* stream, const float* a, size_t a_nbytes, co
     hipError_t e;
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
-        e = mcc::launch_gemm_tn_f32(s, a, b, c, (int)k, (int)m, (int)n, temp, g_contraction_mode.load(), 0, nullptr,
+        e = mcc::launch_gemm_tn_f32(s, a, b, c, (int)k, (int)m, (int)n, temp, g_contraction_mode, 0, nullptr,
                                     sync_words);
     }
     if (temp) {

@@ -836,35 +836,59 @@ DeviceState* current_device_state(hipError_t* err) {
 // Polls (about 0.25 us each) a workgroup spends on one wait before it gives up: roughly four
 // seconds, far above any wait a healthy launch can see.
 constexpr unsigned kDefaultSpinLimit = 1u << 24;
-static std::atomic<unsigned> g_spin_limit{kDefaultSpinLimit};
+// The test aids below belong to the calling thread: a thread that never sets them runs on the
+// defaults whatever other threads do, and no setting can change under a running call.
+static thread_local unsigned g_spin_limit = kDefaultSpinLimit;
 
 // Which tiles a strip launch uses: 0 the wide ones where they keep the device busy, 1 the wide ones
 // whenever the shape allows them, 2 never (tests compare the two kernels).
-static std::atomic<int> g_wide_mode{0};
+static thread_local int g_wide_mode = 0;
 // Test aid: the wide kernel's grid is held to this many workgroups (0: what the device holds), so
 // that small layers run in several passes and park tiles.
-static std::atomic<int> g_wide_grid_cap{0};
+static thread_local int g_wide_grid_cap = 0;
 void set_fused_strip_wide_mode(int mode, int grid_cap) {
-    g_wide_mode.store(mode >= 0 && mode <= 2 ? mode : 0);
-    g_wide_grid_cap.store(grid_cap > 0 ? grid_cap : 0);
+    g_wide_mode = mode >= 0 && mode <= 2 ? mode : 0;
+    g_wide_grid_cap = grid_cap > 0 ? grid_cap : 0;
 }
 
-unsigned fused_strip_spin_limit() { return g_spin_limit.load(); }
-void set_fused_strip_spin_limit(unsigned spins) { g_spin_limit.store(spins ? spins : kDefaultSpinLimit); }
+unsigned fused_strip_spin_limit() { return g_spin_limit; }
+void set_fused_strip_spin_limit(unsigned spins) { g_spin_limit = spins ? spins : kDefaultSpinLimit; }
 
 bool fused_strip_supports(size_t in_features, size_t out_features, size_t batch) {
     return batch > 0 && in_features >= kTile && out_features >= kTile && in_features % kTile == 0 &&
            out_features % kTile == 0 && in_features <= (size_t(1) << 31) / out_features;  // 32-bit element offsets
 }
 
-// Slots for parked tiles of the wide kernel: layers of more than 256 wide tiles -- more than one
-// pass of the persistent grid on a 256-CU device, so that strips can straddle passes -- get two
-// slots for each of the tiles_per_strip - 1 workgroups that may park (1 MiB per 4 slots).
-static size_t park_bytes(size_t in_features, size_t out_features, size_t batch) {
+// Workgroups of the wide kernel the current device holds at once (one per CU); 256 when no device
+// can be asked (a size query on a machine without a GPU).
+static long wide_device_capacity() {
+    static std::atomic<long> cached[kMaxDevices];
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    long c = cached[device].load();
+    if (c > 0) return c;
+    int cus = 0, per_cu = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0 ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fused_strip_wide_kernel<false>, kWideThreads, 0) != hipSuccess ||
+        per_cu <= 0) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    c = (long)cus * per_cu;
+    cached[device].store(c);
+    return c;
+}
+
+// Slots for parked tiles of the wide kernel: layers of more wide tiles than one pass of the
+// persistent grid holds (`capacity` workgroups), so that strips can straddle passes, get two slots
+// for each of the tiles_per_strip - 1 workgroups that may park (1 MiB per 4 slots).
+static size_t park_bytes(size_t in_features, size_t out_features, size_t batch, long capacity) {
     if (in_features % kWide || out_features % kWide || batch < (size_t)kBK || batch % kBK) return 0;
     const size_t tiles_x = in_features / kWide, tiles = tiles_x * (out_features / kWide);
-    const int cap = g_wide_grid_cap.load();
-    if (tiles <= (size_t)(cap ? cap : 256) || tiles_x < 2) return 0;
+    if (tiles <= (size_t)capacity || tiles_x < 2) return 0;
     return 2 * (tiles_x - 1) * (size_t)kParkSlotFloats * sizeof(float);
 }
 
@@ -875,7 +899,14 @@ static size_t strip_base_bytes(size_t out_features) {
 
 size_t fused_strip_workspace_nbytes(size_t in_features, size_t out_features, size_t batch) {
     if (!fused_strip_supports(in_features, out_features, batch)) return 0;
-    return strip_base_bytes(out_features) + park_bytes(in_features, out_features, batch);
+    return strip_base_bytes(out_features) + park_bytes(in_features, out_features, batch, wide_device_capacity());
+}
+
+size_t fused_strip_workspace_nbytes_for_grid(size_t in_features, size_t out_features, size_t batch, int grid_cap) {
+    if (!fused_strip_supports(in_features, out_features, batch)) return 0;
+    const long device = wide_device_capacity();
+    const long capacity = grid_cap > 0 && grid_cap < device ? grid_cap : device;
+    return strip_base_bytes(out_features) + park_bytes(in_features, out_features, batch, capacity);
 }
 
 hipError_t fused_strip_take_failures(int* count) {
@@ -892,8 +923,7 @@ hipError_t fused_strip_take_failures(int* count) {
 hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, float* v, const float* grad_out,
                               const float* x, void* workspace, int C, int in_features, int out_features, int tokens,
                               float lr, float lr_scale, float rms_beta, float rms_eps, uint32_t seed,
-                              unsigned spin_limit, bool* busy) {
-    *busy = false;
+                              unsigned spin_limit, size_t workspace_nbytes) {
     const int strips = out_features / kTile;
     StripArgs a;
     a.state = state;
@@ -938,19 +968,17 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     a.failures = dev->failures;
 
     // Tiles of a strip wait for each other, so every workgroup of the launch has to be resident:
-    // a second strip launch running beside this one on another stream could starve both.  Refuse
-    // it (the caller orders the two).  A stream under capture is left alone: what its graph later
-    // runs beside is the caller's to order.
+    // a second strip launch running beside this one on another stream could starve both.  A launch
+    // on another stream than the last one is therefore ordered behind it on the device (the
+    // stream waits for the event recorded after that launch; nothing is allocated, the host does
+    // not wait).  A stream under capture is left alone: what its graph later runs beside is the
+    // caller's to order.
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
     const bool capturing = capture != hipStreamCaptureStatusNone;
     if (!capturing && dev->launched && dev->last_stream != stream) {
-        const hipError_t q = hipEventQuery(dev->last_launch);
-        (void)hipGetLastError();  // "not ready" is an answer here, not a failure to carry along
-        if (q == hipErrorNotReady) {
-            *busy = true;
-            return hipSuccess;
-        }
+        err = hipStreamWaitEvent(stream, dev->last_launch, 0);
+        if (err != hipSuccess) return err;
     }
 
     // the whole grid must be resident at once: size it from what the device can hold
@@ -965,7 +993,8 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     // parked tiles in the workspace a round is any 256 tiles (4096 x 11008: 688 tiles, three
     // rounds for 2.69); without them a round is whole strips (4096 x 4096 is one round of 16 strips
     // of 16 tiles; 4096 x 11008 would be four rounds of five strips of 43 tiles).
-    const int wide_mode = g_wide_mode.load();
+    const int wide_mode = g_wide_mode;
+    const int grid_cap = g_wide_grid_cap;  // read once: sizing and launch agree
     bool parking = false;
     if (wide_mode != 2 && vec_a && in_features % kWide == 0 && out_features % kWide == 0 && tokens >= kBK &&
         tokens % kBK == 0) {
@@ -973,11 +1002,13 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
         int wide_per_cu = 0;
         err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&wide_per_cu, wide, kWideThreads, 0);
         if (err != hipSuccess) return err;
-        const int cap = g_wide_grid_cap.load();
-        const long capacity = cap && cap < (long)cus * wide_per_cu ? cap : (long)cus * wide_per_cu;
+        const long capacity = grid_cap && grid_cap < (long)cus * wide_per_cu ? grid_cap : (long)cus * wide_per_cu;
         const long tiles_x = in_features / kWide, wide_strips = out_features / kWide, tiles = tiles_x * wide_strips;
         if (capacity >= tiles_x) {
-            parking = park_bytes((size_t)in_features, (size_t)out_features, (size_t)tokens) != 0 && tiles > capacity;
+            const size_t park = park_bytes((size_t)in_features, (size_t)out_features, (size_t)tokens, capacity);
+            parking = park != 0;
+            // the caller sized the workspace without the test aid's grid: tiles cannot be parked
+            if (parking && workspace_nbytes < strip_base_bytes((size_t)out_features) + park) return hipErrorInvalidValue;
             const long per_round = parking ? capacity : capacity / tiles_x * tiles_x;
             const long rounds = (tiles + per_round - 1) / per_round;
             if (wide_mode == 1 || tiles * 5 >= rounds * capacity * 4) {
@@ -994,8 +1025,7 @@ hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, 
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0);
     if (err != hipSuccess) return err;
     long capacity = (long)cus * per_cu;
-    if (threads == kWideThreads && g_wide_grid_cap.load() && g_wide_grid_cap.load() < capacity)
-        capacity = g_wide_grid_cap.load();
+    if (threads == kWideThreads && grid_cap && grid_cap < capacity) capacity = grid_cap;
     a.layer_wgs = cus;
     if (capacity < a.tiles_per_strip) return hipErrorLaunchOutOfResources;
     // a whole number of strips per pass of the persistent grid: a strip that straddled two passes

@@ -105,6 +105,11 @@ void mcc_compact_counter_fused_strip_set_tile_mode(int mode, int grid_cap) {
     mcc::set_fused_strip_wide_mode(mode, grid_cap);
 }
 
+size_t mcc_compact_counter_fused_strip_workspace_nbytes_for_grid(size_t in_features, size_t out_features,
+                                                                 size_t batch, int grid_cap) {
+    return mcc::fused_strip_workspace_nbytes_for_grid(in_features, out_features, batch, grid_cap);
+}
+
 void mcc_contraction_spans_set_test_mode(unsigned polls, int start_first) {
     mcc::set_gemm_tn_wide_spans_test_mode(polls, start_first);
 }

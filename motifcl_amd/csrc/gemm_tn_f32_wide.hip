@@ -224,9 +224,10 @@ __global__ void clear_words_kernel(int* words, int n) {
 
 // about 0.9 us per poll: 4 ms before a taker computes a tile alone
 constexpr unsigned kDefaultSpanPolls = 4096;
-std::atomic<unsigned> g_span_polls{kDefaultSpanPolls};
-std::atomic<int> g_span_start_first{0};
-std::atomic<int> g_span_order_override{-1};
+// test aids of the calling thread (other threads keep the defaults)
+thread_local unsigned g_span_polls = kDefaultSpanPolls;
+thread_local int g_span_start_first = 0;
+thread_local int g_span_order_override = -1;
 
 int device_cus() {
     static std::atomic<int> cached[64];
@@ -284,16 +285,16 @@ hipError_t launch_gemm_tn_wide_spans(hipStream_t stream, const float* a, const f
             order = step == tiles_y ? 1 : 2;
         }
     }
-    if (g_span_order_override.load() >= 0) { classes = 0; order = 0; }
+    if (g_span_order_override >= 0) { classes = 0; order = 0; }
     hipLaunchKernelGGL(gemm_tn_wide_spans_kernel, dim3(wgs), dim3(kWideThreads), 0, stream, a, b, out, k, m, n,
-                       tiles_x, tiles_y, words, g_span_polls.load(), g_span_start_first.load(), classes, order);
+                       tiles_x, tiles_y, words, g_span_polls, g_span_start_first, classes, order);
     return hipGetLastError();
 }
 
 void set_gemm_tn_wide_spans_test_mode(unsigned polls, int start_first) {
-    g_span_polls.store(polls == 0xffffffffu ? kDefaultSpanPolls : polls);
-    g_span_start_first.store(start_first & 1);
-    g_span_order_override.store((start_first & 2) ? 0 : -1);
+    g_span_polls = polls == 0xffffffffu ? kDefaultSpanPolls : polls;
+    g_span_start_first = start_first & 1;
+    g_span_order_override = (start_first & 2) ? 0 : -1;
 }
 
 }  // namespace mcc

@@ -236,8 +236,7 @@ __device__ __forceinline__ void wide_accumulate(const float* __restrict__ a, con
           [pa1] "+v"(pa1), [pb0] "+v"(pb0), [pb1] "+v"(pb1), [i] "=&s"(i), [t] "=&s"(tmp), [go] "=&s"(go)
         : [va] "v"(va), [vb] "v"(vb), [va2] "v"(va + 65536u), [vb2] "v"(vb + 65536u), [n] "s"(slabs), [dst] "s"(dst),
           [sa] "s"(sa), [sb] "s"(sb), [ph] "s"(turn)
-        // and m0, which the compiler sets before each of its own uses
-        : "memory", "scc", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242",
+        : "memory", "scc", "m0", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242",
           "v243");
 }
 

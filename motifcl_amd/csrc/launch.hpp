@@ -107,16 +107,21 @@ unsigned fused_strip_spin_limit();
 void set_fused_strip_spin_limit(unsigned spins);
 // Tiles of the strip step: 0 chosen by shape (256 x 256 where their rounds keep the device busy,
 // else 128 x 128), 1 wide whenever the shape allows, 2 never wide.  The result is the same bytes.
-// grid_cap > 0 (a test aid) holds the wide kernel's grid to that many workgroups; it also enters
-// fused_strip_workspace_nbytes, which sizes the slots for parked tiles.
+// grid_cap > 0 (a test aid) holds the wide kernel's grid to that many workgroups, which then park
+// tiles on small layers too: such a launch needs fused_strip_workspace_nbytes_for_grid bytes.
+// Both settings, like the spin limit, belong to the calling thread.
 void set_fused_strip_wide_mode(int mode, int grid_cap);
-// *busy: another strip launch of this process is still running on a different stream of the GPU
-// (nothing was enqueued).  Strip launches that give up a wait raise a per-device count that
-// fused_strip_take_failures reads and clears (the stream must have been synchronised).
+size_t fused_strip_workspace_nbytes_for_grid(size_t in_features, size_t out_features, size_t batch, int grid_cap);
+// A launch on another stream than the previous strip launch of this GPU is ordered behind it on
+// the device (the two would compete for resident workgroups).  Strip launches that give up a wait
+// raise a per-device count that fused_strip_take_failures reads and clears (the stream must have
+// been synchronised).  workspace_nbytes: what the caller lent (checked against the parking slots
+// the launch needs).
 hipError_t launch_fused_strip(hipStream_t stream, uint8_t* state, float* scale, float* v,
                               const float* grad_out, const float* x, void* workspace, int C,
                               int in_features, int out_features, int tokens, float lr, float lr_scale,
-                              float rms_beta, float rms_eps, uint32_t seed, unsigned spin_limit, bool* busy);
+                              float rms_beta, float rms_eps, uint32_t seed, unsigned spin_limit,
+                              size_t workspace_nbytes);
 hipError_t fused_strip_take_failures(int* count);
 
 hipError_t launch_decode_weight(hipStream_t stream, const uint8_t* state, const float* scale,

@@ -58,6 +58,8 @@ SIGNATURES = {
 DIAG_SIGNATURES = {
     "mcc_compact_counter_fused_strip_set_spin_limit": (None, [ctypes.c_uint]),
     "mcc_compact_counter_fused_strip_set_tile_mode": (None, [ctypes.c_int, ctypes.c_int]),
+    "mcc_compact_counter_fused_strip_workspace_nbytes_for_grid": (ctypes.c_size_t, [ctypes.c_size_t, ctypes.c_size_t,
+                                                                                    ctypes.c_size_t, ctypes.c_int]),
     "mcc_contraction_spans_set_test_mode": (None, [ctypes.c_uint, ctypes.c_int]),
     "mcc_clock_probe": (ctypes.c_int, [_vp, _vp, _sz, ctypes.c_double]),
     "mcc_wall_clock_khz": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int)]),

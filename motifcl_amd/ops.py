@@ -114,9 +114,8 @@ def fused_strip_workspace_nbytes(in_features, out_features, batch):
 def fused_check(workspace, in_features, out_features, batch):
     """Waits for the stream and raises MccError if a strip-workspace step gave up a wait."""
     L = _lib.load()
-    _lib.check(L.mcc_compact_counter_fused_check(
-        _stream(), workspace.data_ptr(), workspace.numel() * workspace.element_size(),
-        in_features, out_features, batch))
+    ptr, nbytes = (0, 0) if workspace is None else (workspace.data_ptr(), workspace.numel() * workspace.element_size())
+    _lib.check(L.mcc_compact_counter_fused_check(_stream(), ptr, nbytes, in_features, out_features, batch))
 
 
 def apply_update_fused(state, scale, v, grad_out, x, workspace, C, lr, lr_scale, rms_beta, rms_eps,

@@ -3,6 +3,10 @@
 cfg4: one [4096, 4096] tensor of the layer at the full 32768 tokens -- the contraction within
 1e-4 of the oracle's sequential fp32 sum, state / scale / v bit-exact given the GPU's own gradient,
 and the fraction of counters that land on another code than the oracle's reported and bounded.
+The 11008-wide shapes of the layer (the equal-spans contraction and the four-wave update kernel
+together) meet the oracle the same way at 16384 tokens -- half the config's token count, which
+halves the oracle's 22 s per case and takes the same kernels -- through the full workspace, and
+the strip workspace (parked tiles, no gradient buffer) must give the full workspace's bytes.
 cfg3: one tensor of each shape of the 224 at full size, update-only, bit-exact.
 The oracle needs a few seconds per case on 16 threads."""
 import numpy as np
@@ -47,6 +51,43 @@ def test_cfg4_tensor_at_32768_tokens_against_the_oracle(ops, oracle, lr_scale):
     print("    scale: max abs diff %.2e of max %.2e; v: max rel diff %.2e" % (
         np.abs(got[1] - e_scale).max(), np.abs(e_scale).max(), (np.abs(got[2] - e_v) / e_v).max()))
     assert np.abs(got[1] - e_scale).max() <= 1e-5 * np.abs(e_scale).max()
+    np.testing.assert_allclose(got[2], e_v, rtol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(11008, 4096), (4096, 11008)], ids=lambda s: "%dx%d" % s)
+def test_cfg4_wide_tensors_at_16384_tokens_against_the_oracle(ops, oracle, shape):
+    tokens = 16384
+    n_out, n_in = shape
+    print("cfg4 wide tensor", shape, flush=True)
+    x = ops.fill_normal(torch.empty(tokens, n_in, device="cuda"), 111, 1.0)
+    dy = ops.fill_normal(torch.empty(tokens, n_out, device="cuda"), 112, 0.01)
+    st = make_state(ops, n_out, n_in, 113)
+    h0 = [t.cpu().numpy().copy() for t in st]
+    full_nbytes = ops.fused_workspace_nbytes(n_in, n_out, tokens)
+    assert full_nbytes > n_out * n_in * 4   # with the hand-off words of the equal-spans contraction
+    ws = torch.empty(full_nbytes, dtype=torch.uint8, device="cuda")
+    ops.apply_update_fused(st[0], st[1], st[2], dy, x, ws, C, LR, 0.0, BETA, EPS, 4343)
+    torch.cuda.synchronize()
+    got = [t.cpu().numpy() for t in st]
+    g_gpu = ws.view(torch.float32)[: n_out * n_in].view(n_out, n_in).cpu().numpy()
+    # the same step with no gradient buffer
+    st2 = [torch.from_numpy(a).cuda() for a in h0]
+    strip_nbytes = ops.fused_strip_workspace_nbytes(n_in, n_out, tokens)
+    assert 0 < strip_nbytes < full_nbytes // 4
+    ws2 = torch.empty(strip_nbytes, dtype=torch.uint8, device="cuda")
+    ops.apply_update_fused(st2[0], st2[1], st2[2], dy, x, ws2, C, LR, 0.0, BETA, EPS, 4343)
+    ops.fused_check(ws2, n_in, n_out, tokens)
+    for a, b in zip(st2, got):
+        assert np.array_equal(a.cpu().numpy(), b), "strip workspace and full workspace differ"
+    e_state, e_scale, e_v, g_seq = oracle.update_fused(h0[0], h0[1], h0[2], dy.cpu().numpy(), x.cpu().numpy(), C, LR,
+                                                      0.0, BETA, EPS, 4343)
+    rel = np.abs(g_gpu - g_seq).max() / np.abs(g_seq).max()
+    assert rel <= 1e-4, rel
+    x_state, x_scale, x_v = oracle.update_dense(h0[0], h0[1], h0[2], g_gpu, C, LR, 0.0, BETA, EPS, 4343)
+    assert np.array_equal(got[0], x_state) and np.array_equal(got[1], x_scale) and np.array_equal(got[2], x_v)
+    flips = float((oracle.unpack_codes(got[0]) != oracle.unpack_codes(e_state)).mean())
+    print("cfg4 [%d,%d]@%d: max|dG|/max|G| = %.2e, flip fraction = %.2e" % (n_out, n_in, tokens, rel, flips))
+    assert flips <= 1e-4
     np.testing.assert_allclose(got[2], e_v, rtol=1e-5)
 
 

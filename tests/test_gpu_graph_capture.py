@@ -82,3 +82,45 @@ def test_captured_steps_replay_like_eager(ops, path, shapes):
                 assert torch.equal(got, want), "replay %d differs from the eager step" % r
     if path == "strip":
         ops.fused_check(ws[: nbytes[0]], shapes[0][1], shapes[0][2], shapes[0][0])
+
+
+@pytest.mark.parametrize("shape", [(256, 512, 256, 11), (32, 4096, 4096, 11)], ids=["full", "strip"])
+def test_static_workspace_step_is_capturable_and_allocates_nothing(ops, shape):
+    # the entry point without a workspace argument, after one eager call on this GPU (the call that
+    # resolves the static array's address): captured, replayed three times against eager steps, with
+    # the device's free memory unchanged over capture and replays
+    n, n_in, n_out, C = shape
+    if shape[1] == 4096:  # 64 MiB of gradient do not fit the static array: the strip path runs
+        assert ops.fused_workspace_nbytes(n_in, n_out, n) > (32 << 20)
+    st, sc, v, x, dy = fresh(shape, 31)
+
+    def step(t, seed):
+        ops.apply_update_fused_static(t[0], t[1], t[2], t[4], t[3], C, 3e-3, 0.0, 0.9, 1e-3, seed)
+
+    eager = [dev(a) for a in (st, sc, v, x, dy)]
+    snapshots = []
+    for r in range(3):
+        step(eager, 5)
+        torch.cuda.synchronize()
+        snapshots.append([t.clone() for t in eager[:3]])
+    graphed = [dev(a) for a in (st, sc, v, x, dy)]
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        warm = [dev(a) for a in (st, sc, v, x, dy)]
+        step(warm, 5)                                   # the first call on the capture stream is eager
+        torch.cuda.synchronize()
+        del warm
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        with torch.cuda.graph(graph, stream=side):
+            step(graphed, 5)
+    torch.cuda.synchronize()
+    for r in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(graphed[:3], snapshots[r]):
+            assert torch.equal(got, want), "replay %d differs from the eager step" % r
+    # torch's own allocator may hand memory back meanwhile; the library must not have taken any
+    assert torch.cuda.mem_get_info()[0] >= free_before
+    ops.fused_check(None, n_in, n_out, n)
