@@ -9,12 +9,18 @@ fused update of all seven tensors.  The same JSON line carries
   "small_configs"  BASELINE configs 0-2 (one 288x288 layer; the 15M- and the 110M-shaped steps):
                    fused step on the GPU, the same step on the CPU, and the share of counters that
                    land on a different code,
+  "fused_strip"    the same cfg4 step with no weight-sized buffer (update applied from the
+                   contraction's accumulators; 24 MB of workspace instead of 180 MB),
+  "reference_microbench"  the reference's own published benchmark shape (in 1024, out 256, 8 tokens,
+                   C = 3): wall p50 / min / p99 of 50 dispatch+wait runs after 5 warm-ups for the fused
+                   update, decode and grad_x, beside the reference's RX 580 figures (context only: the
+                   shape is launch-bound),
   "cpu_baseline"   the CPU restatement timed on this box's host cores on a bounded sample,
   "parity"         correctness gates measured in the same run.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg0|cfg1|cfg2|cfg4]
                     [--fused-path workspace|strip] [--batched] [--graph]
-                    [--no-update-only] [--no-small] [--no-by-row-length] [--no-cpu] [--no-clock]
+                    [--no-update-only] [--no-strip] [--no-small] [--no-by-row-length] [--no-cpu] [--no-clock]
 
 Inputs are synthetic, from the library's counter-based generator (lowbias32 of element index
 and stream id -> Box-Muller; mcc_fill_normal_f32 / mcc_fill_counter_state_u8), seed 0:
@@ -96,13 +102,25 @@ def make_state(ops, n_out, n_in):
 
 
 def cpu_model():
+    """Everything /proc/cpuinfo says about the first processor's identity, and how many there are."""
+    want = ("model name", "vendor_id", "cpu family", "model", "stepping", "cpu MHz", "cache size")
+    got, count = {}, 0
     try:
         for line in open("/proc/cpuinfo"):
-            if line.startswith("model name"):
-                return line.split(":", 1)[1].strip()
+            if ":" not in line:
+                continue
+            key, val = [t.strip() for t in line.split(":", 1)]
+            if key == "processor":
+                count += 1
+            elif key in want and key not in got:
+                got[key] = val
     except OSError:
-        pass
-    return "unknown"
+        return "unknown"
+    if not got:
+        return "unknown"
+    return "%s (%s family %s model %s stepping %s, %s MHz, cache %s; %d logical processors visible)" % (
+        got.get("model name", "?"), got.get("vendor_id", "?"), got.get("cpu family", "?"), got.get("model", "?"),
+        got.get("stepping", "?"), got.get("cpu MHz", "?"), got.get("cache size", "?"), count)
 
 
 # ------------------------------------------------------------------------------ timing
@@ -534,20 +552,102 @@ def small_config(L, ops, name, steps, warmup, with_cpu):
                     out["cpu_one_thread"] = {"seconds_per_step": time.perf_counter() - t1, "threads": 1}
                 finally:
                     oracle.set_num_threads(threads)
-        L.mcc_profiler_reset()
-        L.mcc_profiler_enable(1)
+        # timed with nothing else on the stream; the kernels' own durations come from a second pass
+        # with the library's event bracketing on (at 50 us a step the events are not free)
         k_steps = max(steps, 10)
         mean_ms, med_ms = time_steps(w.step, k_steps, warmup)
+        L.mcc_profiler_reset()
+        L.mcc_profiler_enable(1)
+        time_steps(w.step, k_steps, 0)
         gemm_ms, _ = query(L, "gemm_tn_f32")
         L.mcc_profiler_enable(0)
         L.mcc_profiler_reset()
-        tf = w.flops * (k_steps + warmup) / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else None
+        tf = w.flops * k_steps / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else None
         out[mode] = {"ms_per_step": mean_ms, "median_ms_per_step": med_ms, "gparam_per_s": w.params / (mean_ms * 1e-3) / 1e9,
                      "contraction_tflops": tf, "contraction_mfma_frac": tf / PEAK_MFMA_F32_TFLOPS if tf else None,
                      "step_mfma_frac": w.flops / (mean_ms * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS}
         out["params"], out["tensors"], out["tokens"] = w.params, len(w.tensors), w.tokens
+        if mode == "batched":
+            out["update_only"] = small_update_only(ops, w, steps, with_cpu)
         del w
         torch.cuda.empty_cache()
+    return out
+
+
+def small_update_only(ops, w, steps, with_cpu):
+    """The update-only step of a small config: a precomputed G ~ N(0, 0.01) per tensor, one batched
+    call on the GPU and the same step on the CPU restatement from the same snapshot."""
+    import numpy as np
+    import torch
+    grads = [normal(ops, (n_out, n_in), 0.01) for (_, _, _, n_out, n_in) in w.tensors]
+    batch = ops.UpdateBatch([(st[0], st[1], st[2], g) for (st, _, _, _, _), g in zip(w.tensors, grads)], LR,
+                            [777 + k for k in range(len(w.tensors))])
+    out = {}
+    if with_cpu:
+        from oracle import counter_oracle as oracle
+        snap = w.snapshot()
+        ops.apply_update_dense_batched(batch, C, LR_SCALE, BETA, EPS)
+        torch.cuda.synchronize()
+        after = w.snapshot()
+        host_g = [g.cpu().numpy() for g in grads]
+        t0 = time.perf_counter()
+        exp = [oracle.update_dense(snap[k][0], snap[k][1], snap[k][2], host_g[k], C, LR, LR_SCALE, BETA, EPS, 777 + k)
+               for k in range(len(w.tensors))]
+        cpu_s = time.perf_counter() - t0
+        out["cpu"] = {"seconds_per_step": cpu_s, "gparam_per_s": w.params / cpu_s / 1e9, "threads": oracle.num_threads(),
+                      "sample": "the whole step, every tensor, once"}
+        out["state_scale_v_bit_exact_vs_cpu"] = bool(all(
+            np.array_equal(a, b) for k in range(len(w.tensors)) for a, b in zip(after[k], exp[k])))
+    mean_ms, med_ms = time_steps(lambda i: ops.apply_update_dense_batched(batch, C, LR_SCALE, BETA, EPS), max(steps, 10), 2)
+    out["gpu"] = {"ms_per_step": mean_ms, "median_ms_per_step": med_ms, "gparam_per_s": w.params / (mean_ms * 1e-3) / 1e9,
+                  "hbm_frac": BYTES_PER_PARAM * w.params / (med_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    return out
+
+
+# ------------------------------------------------------------------------------ the reference's own benchmark shape
+def reference_microbench(ops):
+    """in 1024, out 256, 8 tokens, C = 3: wall time of one dispatch + wait, median of 50 runs after 5
+    warm-ups, for the fused update, decode and grad_x -- the shape and method of the reference's
+    published figures (benchmarks/bench_vulkan_perf.cpp:8-10,862-911).  Launch-bound: it says what a
+    call costs, nothing about the kernels."""
+    import torch
+    n, n_in, n_out, c = 8, 1024, 256, 3
+    state = ops.fill_counter_state(torch.empty(n_out * n_in // 4 * 3, dtype=torch.uint8, device="cuda"), _stream_id(), 15)
+    scale = torch.full((n_out,), math.sqrt(3.0 / (2.0 * n_in)), dtype=torch.float32, device="cuda")
+    v = torch.zeros(n_out, dtype=torch.float32, device="cuda")
+    x = normal(ops, (n, n_in), 1.0)
+    dy = normal(ops, (n, n_out), 0.01)
+    ws = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, n), dtype=torch.uint8, device="cuda")
+    w_out = torch.empty(n_out, n_in, device="cuda")
+    gx = torch.empty(n, n_in, device="cuda")
+    seed = [0]
+
+    def update():
+        seed[0] += 1
+        ops.apply_update_fused(state, scale, v, dy, x, ws, c, 3e-3, 0.0, 0.9, 1e-3, 12345 + seed[0])
+
+    ops_by_name = {
+        "fused_update": update,
+        "decode_weight": lambda: ops.decode_weight(state, scale, c, n_in, n_out, out=w_out),
+        "backward_input": lambda: ops.backward_input(dy, state, scale, c, n_in, out=gx),
+    }
+    published = {"fused_update": 608.6, "decode_weight": 188.3, "backward_input": 501.2}
+    out = {"shape": "in1024_out256_N8, C=3", "method": "wall time of dispatch + wait, 50 runs after 5 warm-ups",
+           "note": "the reference's figures are from one Radeon RX 580 (Vulkan wall p50, reports/vulkan-perf/*.json:7); "
+                   "context only, the shape is launch-bound"}
+    for name, fn in ops_by_name.items():
+        for _ in range(5):
+            fn()
+            torch.cuda.synchronize()
+        us = []
+        for _ in range(50):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            us.append((time.perf_counter() - t0) * 1e6)
+        us.sort()
+        out[name] = {"wall_us_p50": statistics.median(us), "wall_us_min": us[0], "wall_us_p99": us[-1],
+                     "reference_rx580_wall_us_p50": published[name]}
     return out
 
 
@@ -636,6 +736,7 @@ def main():
     ap.add_argument("--batched", action="store_true",
                     help="fused leg through mcc_compact_counter_apply_update_fused_batched (one call per step)")
     ap.add_argument("--no-update-only", action="store_true", help="skip the cfg3 update-only leg")
+    ap.add_argument("--no-strip", action="store_true", help="skip the strip-workspace leg of the cfg4 step")
     ap.add_argument("--no-small", action="store_true", help="skip the cfg0-cfg2 legs")
     ap.add_argument("--no-by-row-length", action="store_true",
                     help="skip the update-only sub-legs by row length (counter runs want the cfg3 launches only)")
@@ -700,6 +801,16 @@ def main():
             line["parity"] = {"counter_flip_mismatch_fraction_vs_sequential_sum": small["counter_flip_mismatch_fraction_vs_cpu"]}
     w = None
     torch.cuda.empty_cache()
+    if args.fused_path == "workspace" and args.workload == "cfg4" and not args.no_strip:
+        # the same step with no weight-sized buffer: same workload and seeds, its own roofline
+        strip, _ = bench_fused(L, ops, args.workload, args.steps, args.warmup, "strip")
+        line["fused_strip"] = {"ms_per_step": strip["ms_per_step"], "median_ms_per_step": strip["median_ms_per_step"],
+                               "value": strip["value"], "unit": "Gparam/s", "roofline": strip["roofline"],
+                               "workspace_bytes": strip["workspace_bytes"],
+                               "fused_check": "ok: no strip step gave up a wait"}
+        torch.cuda.empty_cache()
+    if not args.no_extras:
+        line["reference_microbench"] = reference_microbench(ops)
     if args.fused_path == "workspace" and not args.no_extras:
         # the same step with the optional split-bf16 contraction (six bf16 matrix passes per
         # product, binary32 accuracy), reported beside the headline, which stays on the fp32

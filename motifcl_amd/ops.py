@@ -163,9 +163,9 @@ def matmul_transpose_a(a, b, out=None):
     return out
 
 
-def decode_weight(state, scale, C, in_features, out_features):
+def decode_weight(state, scale, C, in_features, out_features, out=None):
     L = _lib.load()
-    w = torch.empty((out_features, in_features), dtype=torch.float32, device=state.device)
+    w = out if out is not None else torch.empty((out_features, in_features), dtype=torch.float32, device=state.device)
     _lib.check(L.mcc_compact_counter_decode_weight(
         _stream(), *_buf(state, torch.uint8), *_buf(scale, torch.float32), *_buf(w, torch.float32),
         in_features, out_features, C))
