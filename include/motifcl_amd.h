@@ -220,10 +220,22 @@ int mcc_compact_counter_apply_update_fused_static(
  * of a caller that keeps every layer's grad_out and x alive until the end of
  * its backward pass, which is equivalent because no layer's update reads
  * another layer's state.  state, scale and v come out bit-identical to calling
- * mcc_compact_counter_apply_update_fused per tensor with a full workspace.
+ * mcc_compact_counter_apply_update_fused per tensor with a full workspace --
+ * except for a list that runs as equal spans: when every layer's sides are
+ * multiples of 256, every token count a multiple of 16 and the list holds at
+ * least 512 tiles of 256 x 256 (the 110M-shaped model: 1296), the contractions
+ * of the whole list are one launch in which every workgroup gets an equal share
+ * of the list's tiles and tokens, with no token chunks: each gradient is then
+ * the unchunked token-order sum (the reference's order up to pairing), state,
+ * scale and v are exact for that gradient, and they equal the per-tensor call's
+ * wherever that call does not split the tokens into chunks and differ from it
+ * by the rounding of its chunk sums elsewhere (counter-flip fraction ~1e-6).
+ * Such a list needs 16-byte aligned grad_out and x.
  * `workspace` (256-byte aligned) holds
  * mcc_compact_counter_fused_batched_workspace_nbytes(tensors, n) bytes: the
- * per-tensor workspaces, each rounded up to 256 bytes, one after the other.
+ * per-tensor workspaces, each rounded up to 256 bytes, one after the other (as
+ * equal spans: out * in floats per tensor plus 1 KiB; the size depends on the
+ * calling thread's contraction mode, so query it in the mode the call runs in).
  * Under MCC_CONTRACTION_BF16X6 the tensors are processed one by one.
  */
 typedef struct mcc_fused_tensor {

@@ -447,18 +447,52 @@ int mcc_compact_counter_apply_update_fused(void* stream, uint8_t* state, size_t 
                              rms_beta, rms_eps, seed);
 }
 
+// A list whose layers all sit on whole 256 x 256 tiles (and hold enough of them) is contracted as
+// equal spans of the whole list, group of at most kSpanGroup tensors by group: one launch per
+// group, no token chunks, a gradient of out * in floats per tensor.  Decided from the shapes (and
+// the calling thread's contraction mode), so the size query and the call agree.
+constexpr size_t kSpanGroup = 96;
+static size_t span_groups(size_t n) { return (n + kSpanGroup - 1) / kSpanGroup; }
+static void span_group_range(size_t n, size_t g, size_t* begin, size_t* end) {
+    const size_t groups = span_groups(n), base = n / groups, rem = n % groups;
+    *begin = g * base + (g < rem ? g : rem);
+    *end = *begin + base + (g < rem ? 1 : 0);
+}
+static bool fused_batched_as_spans(const mcc_fused_tensor* tensors, size_t n) {
+    if (g_contraction_mode != MCC_CONTRACTION_FP32 || n == 0) return false;
+    std::vector<mcc::GemmTnJob> jobs(n);
+    for (size_t i = 0; i < n; ++i) {
+        const mcc_fused_tensor& t = tensors[i];
+        if (t.batch == 0 || t.batch > kIntMax || t.in_features == 0 || t.in_features > kIntMax || t.out_features == 0 ||
+            t.out_features > kIntMax)
+            return false;
+        jobs[i].a = nullptr; jobs[i].b = nullptr; jobs[i].out = nullptr;
+        jobs[i].k = (int)t.batch; jobs[i].m = (int)t.out_features; jobs[i].n = (int)t.in_features;
+    }
+    for (size_t g = 0; g < span_groups(n); ++g) {
+        size_t b, e;
+        span_group_range(n, g, &b, &e);
+        if (!mcc::gemm_tn_spans_group_applies(jobs.data() + b, e - b)) return false;
+    }
+    return true;
+}
+constexpr size_t kSpanWordsBytes = 1024;  // kWideSpanWorkgroups hand-off words behind the gradients
+
 // Where tensor i's slices start in a batched fused workspace: each tensor gets what
-// mcc_compact_counter_fused_workspace_nbytes asks for, rounded up to 256 bytes.
-static size_t fused_batched_region(const mcc_fused_tensor& t) {
+// mcc_compact_counter_fused_workspace_nbytes asks for (as equal spans: its gradient alone), rounded
+// up to 256 bytes.
+static size_t fused_batched_region(const mcc_fused_tensor& t, bool spans) {
+    if (spans) return (t.out_features * t.in_features * sizeof(float) + 255) / 256 * 256;
     const size_t full = mcc_compact_counter_fused_workspace_nbytes(t.in_features, t.out_features, t.batch);
     return full == 0 ? 0 : (full + 255) / 256 * 256;
 }
 
 size_t mcc_compact_counter_fused_batched_workspace_nbytes(const mcc_fused_tensor* tensors, size_t n_tensors) {
     if (!tensors) return 0;
-    size_t total = 0;
+    const bool spans = fused_batched_as_spans(tensors, n_tensors);
+    size_t total = spans ? kSpanWordsBytes : 0;
     for (size_t i = 0; i < n_tensors; ++i) {
-        const size_t r = fused_batched_region(tensors[i]);
+        const size_t r = fused_batched_region(tensors[i], spans);
         if (r == 0 || r > std::numeric_limits<size_t>::max() - total) return 0;
         total += r;
     }
@@ -477,6 +511,7 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
     if (need == 0) return fail(MCC_E_INVALID, "compact-counter fused update requires non-zero dimensions");
     if (workspace_nbytes < need) return fail(MCC_E_INVALID, "compact-counter fused update workspace is too small");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool spans = fused_batched_as_spans(tensors, n_tensors);
     std::vector<mcc::GemmTnJob> jobs(n_tensors);
     std::vector<mcc::UpdateTensor> upd(n_tensors);
     uint8_t* ws = static_cast<uint8_t*>(workspace);
@@ -498,6 +533,9 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
             rc = fail(MCC_E_INVALID, "compact-counter fused update activation buffer is too small");
         else if (reinterpret_cast<uintptr_t>(t.grad_out) % alignof(float) || reinterpret_cast<uintptr_t>(t.x) % alignof(float))
             rc = fail(MCC_E_INVALID, "compact-counter fused update float buffers must be 4-byte aligned");
+        else if (spans && (reinterpret_cast<uintptr_t>(t.grad_out) % 16 || reinterpret_cast<uintptr_t>(t.x) % 16))
+            rc = fail(MCC_E_INVALID, "compact-counter batched fused update of a list of 256-multiple layers requires "
+                                     "16-byte aligned grad_out and x");
         if (rc == MCC_OK) {
             // the state side is checked as for the update-only step, with the tensor's region as gradient
             const mcc_counter_tensor c = {t.state, t.state_nbytes, t.scale, t.scale_nbytes, t.v, t.v_nbytes,
@@ -517,12 +555,13 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
         jobs[i].m = (int)t.out_features;
         jobs[i].n = (int)t.in_features;
         // the region ends with the hand-off words of a shape that uses them
-        jobs[i].sync_words = mcc::gemm_tn_sync_nbytes(jobs[i].k, jobs[i].m, jobs[i].n)
+        jobs[i].sync_words = !spans && mcc::gemm_tn_sync_nbytes(jobs[i].k, jobs[i].m, jobs[i].n)
                                  ? reinterpret_cast<int*>(jobs[i].out + mcc::gemm_tn_slices(jobs[i].k, jobs[i].m, jobs[i].n) *
                                                                            t.out_features * t.in_features)
                                  : nullptr;
-        ws += fused_batched_region(t);
+        ws += fused_batched_region(t, spans);
     }
+    int* span_words = reinterpret_cast<int*>(ws);  // behind the last region (equal spans only)
     if (n_tensors > 1) {
         std::vector<const void*> states(n_tensors);
         for (size_t i = 0; i < n_tensors; ++i) states[i] = tensors[i].state;
@@ -535,7 +574,7 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
         ws = static_cast<uint8_t*>(workspace);
         for (size_t i = 0; i < n_tensors; ++i) {
             const mcc_fused_tensor& t = tensors[i];
-            const size_t region = fused_batched_region(t);
+            const size_t region = fused_batched_region(t, false);
             const int rc = mcc_compact_counter_apply_update_fused(
                 stream, t.state, t.state_nbytes, t.scale, t.scale_nbytes, t.v, t.v_nbytes, t.grad_out, t.grad_out_nbytes,
                 t.x, t.x_nbytes, ws, region, C, t.in_features, t.out_features, t.batch, t.lr, lr_scale, rms_beta,
@@ -548,10 +587,18 @@ int mcc_compact_counter_apply_update_fused_batched(void* stream, const mcc_fused
         }
         return MCC_OK;
     }
-    hipError_t e;
+    hipError_t e = hipSuccess;
     {
         ScopedKernelTimer timer("gemm_tn_f32", s);
-        e = mcc::launch_gemm_tn_group(s, jobs.data(), n_tensors);
+        if (spans) {
+            for (size_t g = 0; g < span_groups(n_tensors) && e == hipSuccess; ++g) {
+                size_t b, en;
+                span_group_range(n_tensors, g, &b, &en);
+                e = mcc::launch_gemm_tn_wide_spans_group(s, jobs.data() + b, en - b, span_words);
+            }
+        } else {
+            e = mcc::launch_gemm_tn_group(s, jobs.data(), n_tensors);
+        }
     }
     if (e != hipSuccess) return hip_fail(e, "compact-counter fused update contraction launch failed");
     {

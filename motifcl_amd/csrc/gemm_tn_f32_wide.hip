@@ -217,6 +217,148 @@ MCC_WIDE_KERNEL void gemm_tn_wide_spans_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------- equal spans over a list
+// The same for a list of contractions (the layers of a model whose sides are multiples of 256):
+// the (tile, slab) sequences of all jobs are laid end to end and every workgroup gets an equal
+// span of the whole, so a list of mid-sized layers -- none of which fills the device with 256 x 256
+// tiles on its own -- runs as one launch with no idle round, no token chunks and no slices to add
+// up.  Every output element is still the sum of its tokens in token order.
+struct SpanJob {
+    const float* a;  // [K, M]
+    const float* b;  // [K, N]
+    float* c;        // [M, N]
+    int K, M, N;
+    int slab_begin;  // first slab of this job in the list's sequence
+};
+constexpr int kMaxSpanJobs = 96;
+struct SpanGroupArgs {
+    SpanJob job[kMaxSpanJobs];
+    int n_jobs;
+    int total_slabs;
+    int* words;
+    unsigned spin_limit;
+    int start_first;
+};
+static_assert(sizeof(SpanGroupArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+
+// One piece of a tile: slabs [from, to) of tile `tile` of job `ji`.
+struct SpanPiece {
+    int ji, tile, from, to, spt;
+};
+
+MCC_WIDE_KERNEL void gemm_tn_wide_spans_group_kernel(SpanGroupArgs g) {
+    __shared__ __attribute__((aligned(1024))) float lds[kWideBuffers * kWideSlabFloats + 64];
+    float& verdict = lds[kWideBuffers * kWideSlabFloats];
+    const WideLane t = wide_lane();
+    const int P = gridDim.x;
+    // neighbouring spans on one XCD: they work on neighbouring tiles, which share operand panels
+    int j = (int)blockIdx.x;
+    if ((P & 7) == 0) j = (int)(blockIdx.x & 7u) * (P >> 3) + (int)(blockIdx.x >> 3);
+    const long total = g.total_slabs;
+    const long base = total / P, rem = total % P;
+    const int begin = (int)(j * base + (j < rem ? j : rem));
+    const int end = (int)(begin + base + (j < rem ? 1 : 0));
+
+    // the piece that holds slab `slab` (scalar: kernel arguments and blockIdx only)
+    auto piece_at = [&](int slab, int ji) {
+        while (ji + 1 < g.n_jobs && g.job[ji + 1].slab_begin <= slab) ++ji;
+        SpanPiece p;
+        p.ji = ji;
+        p.spt = g.job[ji].K / kBK;
+        const int local = slab - g.job[ji].slab_begin;
+        p.tile = local / p.spt;
+        p.from = local - p.tile * p.spt;
+        p.to = p.spt;
+        return p;
+    };
+    auto origin = [&](const SpanPiece& p, const SpanJob& job, int& m0, int& n0) {
+        const TileXY xy = band_tile(p.tile, job.N / kWide, job.M / kWide);
+        m0 = xy.y * kWide;
+        n0 = xy.x * kWide;
+    };
+    SpanPiece first = piece_at(begin, 0);
+    SpanPiece last = piece_at(end - 1, first.ji);
+    last.to = end - g.job[last.ji].slab_begin - last.tile * last.spt;  // slabs of the last tile inside the span
+    last.from = 0;
+    // the host makes every span longer than two tiles, so the two are never the same tile
+    const bool has_start = first.from > 0, has_end = last.to < last.spt;
+    WideAcc acc;
+
+    // the partial tile at the end of the span: slabs [0, to), parked in c for workgroup j + 1
+    auto run_end = [&]() {
+        const SpanJob job = g.job[last.ji];
+        int m0, n0;
+        origin(last, job, m0, n0);
+        wide_zero(acc);
+        __syncthreads();
+        wide_accumulate(job.a + m0, job.b + n0, job.M, job.N, last.to * kBK, acc, lds, t);
+        if (t.tid == 0) verdict = word_claim(&g.words[j], kWriting) ? 1.0f : 0.0f;
+        __syncthreads();
+        if (verdict != 0.0f) {  // else the taker has given up and computes the tile alone
+            wide_park(job.c, job.N, m0, n0, acc, t.tid);
+            __builtin_amdgcn_s_waitcnt(0);  // stores acknowledged
+            __syncthreads();
+            if (t.tid == 0) __hip_atomic_store(&g.words[j], kParked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+    };
+    auto run_whole = [&]() {
+        // from the tile after a partial first one up to the tile before a partial last one
+        int slab = begin + (has_start ? first.spt - first.from : 0);
+        const int stop = has_end ? end - last.to : end;
+        int ji = first.ji;
+        while (slab < stop) {
+            const SpanPiece p = piece_at(slab, ji);
+            ji = p.ji;
+            const SpanJob job = g.job[ji];
+            int m0, n0;
+            origin(p, job, m0, n0);
+            wide_zero(acc);
+            __syncthreads();
+            wide_accumulate(job.a + m0, job.b + n0, job.M, job.N, job.K, acc, lds, t);
+            wide_store(job.c, job.N, m0, n0, acc, t);
+            slab += p.spt;
+        }
+    };
+    // the partial tile at the start: slabs [from, spt) on top of what workgroup j - 1 parked
+    auto run_start = [&]() {
+        const SpanJob job = g.job[first.ji];
+        int m0, n0;
+        origin(first, job, m0, n0);
+        if (t.tid == 0) {
+            int* word = &g.words[j - 1];
+            int got = 0;
+            unsigned polls = 0;
+            for (;;) {
+                const int seen = word_load(word);
+                if (seen == kParked) { got = 1; break; }
+                // kWriting: the owner is running and about to finish, whatever the budget says
+                if (seen == 0 && polls >= g.spin_limit && word_claim(word, kAbandoned)) break;
+                __builtin_amdgcn_s_sleep(32);
+                ++polls;
+            }
+            verdict = got ? 1.0f : 0.0f;
+        }
+        __syncthreads();
+        const bool parked = verdict != 0.0f;
+        if (parked) wide_take(job.c, job.N, m0, n0, acc, t.tid); else wide_zero(acc);
+        const int from = parked ? first.from : 0;
+        __syncthreads();
+        wide_accumulate(job.a + (size_t)from * kBK * job.M + m0, job.b + (size_t)from * kBK * job.N + n0, job.M, job.N,
+                        (first.spt - from) * kBK, acc, lds, t);
+        wide_store(job.c, job.N, m0, n0, acc, t);
+    };
+    if (!g.start_first) {
+        if (has_end) run_end();
+        run_whole();
+        if (has_start) run_start();
+    } else {  // test order: every taker arrives before its owner
+        if (has_start) run_start();
+        run_whole();
+        if (has_end) run_end();
+    }
+}
+
 __global__ void clear_words_kernel(int* words, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) words[i] = 0;
@@ -288,6 +430,49 @@ hipError_t launch_gemm_tn_wide_spans(hipStream_t stream, const float* a, const f
     if (g_span_order_override >= 0) { classes = 0; order = 0; }
     hipLaunchKernelGGL(gemm_tn_wide_spans_kernel, dim3(wgs), dim3(kWideThreads), 0, stream, a, b, out, k, m, n,
                        tiles_x, tiles_y, words, g_span_polls, g_span_start_first, classes, order);
+    return hipGetLastError();
+}
+
+// Whether a list of contractions runs as one launch of equal spans: every job on whole 256 x 256
+// tiles and whole slabs, at least two tiles per workgroup over the list, and -- so that a span never
+// begins and ends inside one tile -- spans of at least two tiles of the job with the most tokens.
+// A function of the shapes alone.
+bool gemm_tn_spans_group_applies(const GemmTnJob* jobs, size_t n) {
+    if (n == 0 || n > (size_t)kMaxSpanJobs) return false;
+    long total = 0, tiles = 0, max_spt = 0;
+    for (size_t i = 0; i < n; ++i) {
+        const GemmTnJob& jb = jobs[i];
+        if (jb.m % kWide || jb.n % kWide || jb.k % kBK || jb.k <= 0) return false;
+        const long t = (long)(jb.m / kWide) * (jb.n / kWide), spt = jb.k / kBK;
+        tiles += t;
+        total += t * spt;
+        if (spt > max_spt) max_spt = spt;
+        if (total >= (1L << 31)) return false;
+    }
+    return tiles >= 2L * kWideSpanWorkgroups && total / kWideSpanWorkgroups >= 2 * max_spt;
+}
+
+hipError_t launch_gemm_tn_wide_spans_group(hipStream_t stream, const GemmTnJob* jobs, size_t n, int* words) {
+    if (!gemm_tn_spans_group_applies(jobs, n)) return hipErrorInvalidValue;
+    int wgs = device_cus();
+    if (wgs <= 0 || wgs > kWideSpanWorkgroups) wgs = kWideSpanWorkgroups;
+    SpanGroupArgs g;
+    long total = 0;
+    for (size_t i = 0; i < n; ++i) {
+        const GemmTnJob& jb = jobs[i];
+        if ((reinterpret_cast<uintptr_t>(jb.a) & 15u) || (reinterpret_cast<uintptr_t>(jb.b) & 15u) ||
+            (reinterpret_cast<uintptr_t>(jb.out) & 15u))
+            return hipErrorInvalidValue;
+        g.job[i] = {jb.a, jb.b, jb.out, jb.k, jb.m, jb.n, (int)total};
+        total += (long)(jb.m / kWide) * (jb.n / kWide) * (jb.k / kBK);
+    }
+    g.n_jobs = (int)n;
+    g.total_slabs = (int)total;
+    g.words = words;
+    g.spin_limit = g_span_polls;
+    g.start_first = g_span_start_first;
+    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(kWideSpanWorkgroups), 0, stream, words, kWideSpanWorkgroups);
+    hipLaunchKernelGGL(gemm_tn_wide_spans_group_kernel, dim3(wgs), dim3(kWideThreads), 0, stream, g);
     return hipGetLastError();
 }
 

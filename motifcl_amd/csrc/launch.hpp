@@ -91,6 +91,12 @@ struct GemmTnJob {
     int* sync_words = nullptr;  // as for launch_gemm_tn_f32
 };
 hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_t n);
+// A list whose jobs all sit on whole 256 x 256 tiles and together hold at least two tiles per CU
+// runs as ONE launch of equal spans of the list's (tile, slab) sequence: no token chunks, no slices
+// (every out is m * n floats, the unchunked token-order sum).  `words` holds kWideSpanWorkgroups
+// ints.  a, b and out must be 16-byte aligned.  ..._applies is a function of the shapes alone.
+bool gemm_tn_spans_group_applies(const GemmTnJob* jobs, size_t n);
+hipError_t launch_gemm_tn_wide_spans_group(hipStream_t stream, const GemmTnJob* jobs, size_t n, int* words);
 
 bool gemm_tn_bf16x6_supports(const float* a, const float* b, int k, int m, int n, const GemmTnPlan& plan);
 hipError_t launch_gemm_tn_bf16x6(hipStream_t stream, const float* a, const float* b, float* out,

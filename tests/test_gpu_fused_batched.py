@@ -57,6 +57,81 @@ def test_batched_fused_step_matches_the_per_tensor_entry_point(ops, oracle, name
     torch.cuda.synchronize()
 
 
+def layer_shapes(dim, hidden, layers, tokens):
+    return ([(dim, dim, tokens)] * 4 + [(hidden, dim, tokens)] * 2 + [(dim, hidden, tokens)]) * layers
+
+
+@pytest.fixture()
+def span_mode():
+    """Test aid of the equal-spans contraction: polls before a taker gives up, takers first."""
+    import motifcl_amd
+    L = motifcl_amd.load()
+    yield lambda polls, start_first: L.mcc_contraction_spans_set_test_mode(polls, start_first)
+    L.mcc_contraction_spans_set_test_mode(0xFFFFFFFF, 0)
+
+
+# the 110M-shaped model (12 layers of 768 / 2048: 1296 tiles of 256 x 256) runs as equal spans of the
+# whole list; with 64 tokens the per-tensor call does not chunk either, so the bytes must be equal
+@pytest.mark.parametrize("mode", ["default", "every_hand_off_abandoned", "takers_first"])
+@pytest.mark.parametrize("lr_scale", [0.0, 1e-3])
+def test_list_of_256_multiple_layers_runs_as_equal_spans_with_the_same_bytes(ops, oracle, span_mode, mode, lr_scale):
+    shapes = layer_shapes(768, 2048, 12, 64)
+    host_tensors = build(ops, oracle, shapes, 21)
+    seeds = [999 + 3 * i for i in range(len(shapes))]
+    expect = []
+    for (state, scale, v, dy, x), seed, (n_out, n_in, tokens) in zip(host_tensors, seeds, shapes):
+        d = [dev(t) for t in (state, scale, v, dy, x)]
+        ws = torch.empty(ops.fused_workspace_nbytes(n_in, n_out, tokens), dtype=torch.uint8, device="cuda")
+        ops.apply_update_fused(*d, ws, HP["C"], HP["lr"], lr_scale, HP["rms_beta"], HP["rms_eps"], seed)
+        expect.append([host(t) for t in d[:3]])
+    d_all = [[dev(t) for t in tensor] for tensor in host_tensors]
+    batch = ops.FusedBatch([tuple(d) for d in d_all], HP["lr"], seeds)
+    need = batch.workspace_nbytes()
+    assert need == sum((o * i * 4 + 255) // 256 * 256 for (o, i, _) in shapes) + 1024   # a gradient per tensor, no slices
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    if mode == "every_hand_off_abandoned":
+        span_mode(0, 1)
+    elif mode == "takers_first":
+        span_mode(0xFFFFFFFF, 1)
+    print("equal spans over a list,", mode, flush=True)
+    ops.apply_update_fused_batched(batch, ws, HP["C"], lr_scale, HP["rms_beta"], HP["rms_eps"])
+    torch.cuda.synchronize()
+    for d, e in zip(d_all, expect):
+        for got, want in zip(d[:3], e):
+            np.testing.assert_array_equal(host(got), want)
+
+
+def test_equal_spans_over_a_list_against_the_oracle(ops, oracle):
+    # 1024 tokens: the per-tensor call would split them into chunks; the list's gradients are the
+    # unchunked sums.  Each gradient within 1e-4 of the oracle's sequential sum, state / scale / v
+    # exact for the GPU's gradient, counter flips against the sequential-sum oracle counted.
+    shapes = layer_shapes(768, 2048, 12, 1024)
+    host_tensors = build(ops, oracle, shapes, 33)
+    seeds = [4000 + i for i in range(len(shapes))]
+    d_all = [[dev(t) for t in tensor] for tensor in host_tensors]
+    batch = ops.FusedBatch([tuple(d) for d in d_all], HP["lr"], seeds)
+    ws = torch.empty(batch.workspace_nbytes(), dtype=torch.uint8, device="cuda")
+    ops.apply_update_fused_batched(batch, ws, HP["C"], 0.0, HP["rms_beta"], HP["rms_eps"])
+    torch.cuda.synchronize()
+    offset, n_flip, n_all = 0, 0, 0
+    for (state, scale, v, dy, x), seed, (n_out, n_in, tokens), d in zip(host_tensors, seeds, shapes, d_all):
+        g_gpu = ws[offset: offset + n_out * n_in * 4].view(torch.float32).view(n_out, n_in).cpu().numpy()
+        offset += (n_out * n_in * 4 + 255) // 256 * 256
+        e_state, e_scale, e_v, g_seq = oracle.update_fused(state, scale, v, dy, x, HP["C"], HP["lr"], 0.0,
+                                                          HP["rms_beta"], HP["rms_eps"], seed)
+        assert np.abs(g_gpu - g_seq).max() <= 1e-4 * np.abs(g_seq).max()
+        x_state, x_scale, x_v = oracle.update_dense(state, scale, v, g_gpu, HP["C"], HP["lr"], 0.0, HP["rms_beta"],
+                                                    HP["rms_eps"], seed)
+        np.testing.assert_array_equal(host(d[0]), x_state)
+        np.testing.assert_array_equal(host(d[1]), x_scale)
+        np.testing.assert_array_equal(host(d[2]), x_v)
+        diff = oracle.unpack_codes(x_state) != oracle.unpack_codes(e_state)
+        n_flip += int(diff.sum())
+        n_all += diff.size
+    print("equal spans over 84 tensors at 1024 tokens: counter-flip fraction vs the sequential-sum oracle %.2e" % (n_flip / n_all))
+    assert n_flip / n_all <= 1e-4
+
+
 def test_batched_fused_step_validates_its_arguments(ops, oracle):
     from motifcl_amd.lib import MccError
     shapes = [(64, 64, 64), (32, 128, 16)]
