@@ -216,7 +216,22 @@ MCC_HD float div_by_row(float gw, float dn, double rd) {
     return (float)((double)gw * rd);
 }
 
-MCC_HD double row_reciprocal(float dn) { return 1.0 / (double)dn; }
+// rd need not be the correctly rounded reciprocal: with a relative error e_rd the double product is
+// q* (1 + e), |e| <= e_rd + 2^-53, and the argument above goes through for e_rd <= 2^-49.1.  The
+// device takes the hardware's approximate reciprocal through two Newton steps (a few 2^-53; five
+// instructions instead of the twenty-five of a correctly rounded division); dn is in
+// [2^-40, 2^40] wherever rd is used, so nothing needs scaling.
+MCC_HD double row_reciprocal(float dn) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const double d = (double)dn;
+    double r = __builtin_amdgcn_rcp(d);
+    r = __builtin_fma(r, __builtin_fma(-d, r, 1.0), r);
+    r = __builtin_fma(r, __builtin_fma(-d, r, 1.0), r);
+    return r;
+#else
+    return 1.0 / (double)dn;
+#endif
+}
 
 MCC_HD float clamp_f(float x, float lo, float hi) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -271,7 +286,19 @@ struct RowStats {
 
 MCC_HD RowStats finish_row_stats(float sum_sq, float sum_gt, float v_old, float scale_old,
                                  int in_features, float lr_scale, float rms_beta, float rms_eps) {
-    const float gsq = sum_sq / (float)in_features;
+    // a power of two divides exactly like its reciprocal multiplies (one rounding of the same real
+    // number either way), and the reciprocal's bits are its exponent: no division
+    float gsq;
+    if ((in_features & (in_features - 1)) == 0) {
+        int log2_in = 0;
+        while ((1 << log2_in) < in_features) ++log2_in;  // a kernel argument: scalar, a handful of instructions
+        const uint32_t inv_bits = (uint32_t)(127 - log2_in) << 23;
+        float inv;
+        __builtin_memcpy(&inv, &inv_bits, 4);
+        gsq = sum_sq * inv;
+    } else {
+        gsq = sum_sq / (float)in_features;
+    }
     // lr_scale == 0: the product below is +-0 for every finite gs and the scale stays as it is
     // (up to its clamp), so the square root and the division are skipped
     const float gs = lr_scale != 0.0f ? sum_gt / sqrtf((float)in_features) : 0.0f;

@@ -225,9 +225,17 @@ __device__ __forceinline__ float wave_min_nonneg(float a, int lane) { return __u
 
 struct RowCtx {
     TickConsts tc;
-    float ratio;    // s_old / s_new: the rebase factor of the residual counters
-    bool fast_div;  // wave-uniform
+    float s_old, s_new;  // the rebase factor of the residual counters is s_old / s_new
+    bool fast_div;       // wave-uniform
 };
+
+// The rebase factor s_old / s_new; a division, so only where a row needs it (lr_scale != 0, or a
+// scale that sat outside its clamp range).
+__device__ __forceinline__ float rebase_ratio(const RowCtx& rc) { return rc.s_old / rc.s_new; }
+// Whether the scale stays as it is (then the factor is exactly 1); wave-uniform.
+__device__ __forceinline__ bool scale_unchanged(const RowCtx& rc) {
+    return __builtin_amdgcn_readfirstlane(rc.s_old == rc.s_new ? 1 : 0) != 0;
+}
 
 // Tree reduction, row epilogue and commit of v/scale.  `exact_key()` returns the lane's exact
 // magnitude key over the row; it is called (by the whole wave) only when the smallest magnitude
@@ -254,7 +262,8 @@ __device__ __forceinline__ RowCtx finish_row(const BatchArgs& a, const UpdateTen
         t.scale[row] = rs.scale_new;  // commit (kernels/basic.cl:6-9); s_old stays in a register
     }
     RowCtx rc;
-    rc.ratio = s_old / rs.scale_new;
+    rc.s_old = s_old;
+    rc.s_new = rs.scale_new;
     rc.tc.dn = rs.denom;
     rc.tc.rd = row_reciprocal(rs.denom);
     rc.tc.k = a.cd.Cf / rs.scale_new;
@@ -316,7 +325,7 @@ __device__ __forceinline__ void apply_streamed(const UpdateTensor& t, int row, i
     const float* g_row = t.grad_w + (size_t)row * t.in_features;
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
     const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
-    const RebasedCounters c_reb{l.c_f, rc.ratio};
+    const RebasedCounters c_reb{l.c_f, rebase_ratio(rc)};
     for (int gi = group_begin + lane; gi < g_end; gi += kWave) {
         float g[4];
 #pragma unroll
@@ -385,12 +394,11 @@ __device__ __forceinline__ void update_row_resident(const BatchArgs& a, const Up
         return key;
     });
     // without lr_scale the scale only moves when it sits outside its clamp range
-    const bool unit_ratio = __builtin_amdgcn_readfirstlane(rc.ratio == 1.0f ? 1 : 0) != 0;
-    if (!rc.fast_div || (!WITH_GS && !unit_ratio)) {
+    if (!rc.fast_div || (!WITH_GS && !scale_unchanged(rc))) {
         apply_streamed(t, row, lane, rc, luts);
         return;
     }
-    const RebasedCounters rebased{luts.c_f, rc.ratio};
+    const RebasedCounters rebased{luts.c_f, WITH_GS ? rebase_ratio(rc) : 1.0f};
     const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
     // EXACT rows: deltas of the first hash products, wave-uniform per 256-element span and the same
     // for every span with equal bits 16..17 of the element index (a whole row, when it is short):
@@ -491,7 +499,7 @@ __device__ __forceinline__ void update_row_two_pass(const BatchArgs& a, const Up
         apply_streamed(t, row, lane, rc, luts);
         return;
     }
-    const RebasedCounters rebased{luts.c_f, rc.ratio};
+    const RebasedCounters rebased{luts.c_f, rebase_ratio(rc)};
     const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
     for (int c0 = 0; c0 < iters; c0 += kChunk) {
         float4 q[kChunk];
@@ -599,7 +607,10 @@ struct SplitShared {
 
 constexpr int min_waves_split(int j) { return j <= 6 ? 4 : 3; }
 
-template <int J, int W, bool WITH_GS>
+// ALIGNED: rows of a whole number of 256-weight iterations (11008 = 43 * 256): no lane is ever
+// masked, an iteration past the row's end is skipped by the whole wave, and every iteration is an
+// aligned span of the element index, so the first hash products come by addition (hash_delta).
+template <int J, int W, bool WITH_GS, bool ALIGNED>
 __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_split_kernel(BatchArgs a) {
     __shared__ SplitShared sh;
     const int lane = threadIdx.x & (kWave - 1);
@@ -612,16 +623,31 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
     const int j0 = w * J;
     const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    // whether lane's group of iteration j0 + jj exists: per iteration when ALIGNED
+    auto live_at = [&](int jj) {
+        return ALIGNED ? j0 + jj < iters : (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+    };
 
     float4 q[J];
     uint32_t words[J];
 #pragma unroll
     for (int jj = 0; jj < J; ++jj) {
         const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
-        const uint32_t gc = gi < gpr ? gi : gpr - 1;
-        q[jj] = load_grad4_once(g_row + gc);
-        words[jj] = last_row ? load_group_dword_or_tail_once(s_row + 3u * gc, gc == gpr - 1)
-                             : load_group_dword_once(s_row + 3u * gc);
+        if (ALIGNED) {
+            if (j0 + jj < iters) {  // wave-uniform
+                q[jj] = load_grad4_once(g_row + gi);
+                words[jj] = last_row ? load_group_dword_or_tail_once(s_row + 3u * gi, gi == gpr - 1)
+                                     : load_group_dword_once(s_row + 3u * gi);
+            } else {
+                q[jj] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                words[jj] = 0u;
+            }
+        } else {
+            const uint32_t gc = gi < gpr ? gi : gpr - 1;
+            q[jj] = load_grad4_once(g_row + gc);
+            words[jj] = last_row ? load_group_dword_or_tail_once(s_row + 3u * gc, gc == gpr - 1)
+                                 : load_group_dword_once(s_row + 3u * gc);
+        }
     }
     build_luts(sh.luts, a.cd, a.geom);  // while the row is in flight
     // What does not depend on the order happens before the hand-off, in all waves at once: the
@@ -634,7 +660,8 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
     if (kPre) {
 #pragma unroll
         for (int jj = 0; jj < J; ++jj) {
-            const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+            // a skipped iteration holds zeros: +0.0 to the sums, the largest key to the minimum
+            const bool live = ALIGNED || live_at(jj);
             const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
                                 live ? q[jj].w : 0.0f};
             my_key = umin3(my_key, range_key(g[0]), range_key(g[1]));
@@ -667,7 +694,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
             } else {
 #pragma unroll
                 for (int jj = 0; jj < J; ++jj) {
-                    const bool live = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+                    const bool live = live_at(jj);
                     const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
                                         live ? q[jj].w : 0.0f};
                     accumulate<WITH_GS, true>(acc, g, live, words[jj], a.cd);
@@ -690,23 +717,40 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
     }
     __syncthreads();
     RowCtx rc = sh.rc;
-    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24), "+v"(rc.tc.seed_mix), "+v"(rc.tc.rd));  // VGPR operands
+    asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24), "+v"(rc.tc.seed_mix));  // VGPR operands
     const bool fast = __builtin_amdgcn_readfirstlane(sh.fast_div) != 0;
-    const bool unit_ratio = __builtin_amdgcn_readfirstlane(rc.ratio == 1.0f ? 1 : 0) != 0;
-    if (!fast || (!WITH_GS && !unit_ratio)) {
+    if (!fast || (!WITH_GS && !scale_unchanged(rc))) {
         apply_streamed(t, row, lane, rc, sh.luts, j0 * kWave, (j0 + J) * kWave);
         return;
     }
-    const RebasedCounters rebased{sh.luts.c_f, rc.ratio};
+    const RebasedCounters rebased{sh.luts.c_f, WITH_GS ? rebase_ratio(rc) : 1.0f};
     const uint32_t row_elem = (uint32_t)(row + t.first_row) * (uint32_t)t.in_features;
+    uint32_t dv[3] = {0u, 0u, 0u};
+    uint32_t dv_bits = 4u;
 #pragma unroll
     for (int jj = 0; jj < J; ++jj) {
         if (j0 + jj < iters) {  // wave-uniform
             const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
             const float g[4] = {q[jj].x, q[jj].y, q[jj].z, q[jj].w};
-            const uint32_t nw = WITH_GS ? tick_group<true>(words[jj], g, rc.tc, rebased, sh.luts, row_elem + 4u * gi)
-                                        : tick_group<true>(words[jj], g, rc.tc, sh.luts.c_f, sh.luts, row_elem + 4u * gi);
-            if (gi < gpr) store_group_once(s_row + 3u * gi, nw);
+            uint32_t nw;
+            if (ALIGNED) {
+                const uint32_t span = row_elem + 4u * kWave * (uint32_t)(j0 + jj);
+                const uint32_t sbits = (span >> 16) & 3u;  // wave-uniform
+                if (sbits != dv_bits) {
+                    dv_bits = sbits;
+                    dv[0] = hash_delta(sbits, 1);
+                    dv[1] = hash_delta(sbits, 2);
+                    dv[2] = hash_delta(sbits, 3);
+                    asm volatile("" : "+v"(dv[0]), "+v"(dv[1]), "+v"(dv[2]));  // the products stay products
+                }
+                const uint32_t p0 = hash_first(span + 4u * (uint32_t)lane) * kHashMul1;
+                nw = WITH_GS ? tick_group_deltas<true>(words[jj], g, rc.tc, rebased, sh.luts, p0, dv)
+                             : tick_group_deltas<true>(words[jj], g, rc.tc, sh.luts.c_f, sh.luts, p0, dv);
+            } else {
+                nw = WITH_GS ? tick_group<true>(words[jj], g, rc.tc, rebased, sh.luts, row_elem + 4u * gi)
+                             : tick_group<true>(words[jj], g, rc.tc, sh.luts.c_f, sh.luts, row_elem + 4u * gi);
+            }
+            if (ALIGNED || gi < gpr) store_group_once(s_row + 3u * gi, nw);
         }
     }
 }
@@ -744,10 +788,10 @@ hipError_t launch_streamed_variant(hipStream_t stream, const BatchArgs& a) {
     return hipGetLastError();
 }
 
-template <int J, int W, bool WITH_GS>
+template <int J, int W, bool WITH_GS, bool ALIGNED>
 hipError_t launch_split_variant(hipStream_t stream, const BatchArgs& a) {
     const dim3 grid((unsigned)a.t[0].out_features, (unsigned)a.n_tensors);
-    hipLaunchKernelGGL((update_rows_split_kernel<J, W, WITH_GS>), grid, dim3(kWave * W), 0, stream, a);
+    hipLaunchKernelGGL((update_rows_split_kernel<J, W, WITH_GS, ALIGNED>), grid, dim3(kWave * W), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -768,9 +812,10 @@ hipError_t launch_long_variant(hipStream_t stream, const BatchArgs& a) {
 
 constexpr int kLongClass = 2000;
 
-template <int J, int W>
+template <int J, int W, bool ALIGNED>
 hipError_t launch_split(hipStream_t stream, const BatchArgs& a) {
-    return a.lr_scale != 0.0f ? launch_split_variant<J, W, true>(stream, a) : launch_split_variant<J, W, false>(stream, a);
+    return a.lr_scale != 0.0f ? launch_split_variant<J, W, true, ALIGNED>(stream, a)
+                              : launch_split_variant<J, W, false, ALIGNED>(stream, a);
 }
 
 template <int ITERS, bool EXACT>
@@ -806,7 +851,7 @@ int iters_class(const UpdateTensor& t) {
     // once; every other long row takes the two-pass wave (measured at 4096 rows: 5120-wide 639
     // against 425 Gweights/s for the cooperating waves, 8192-wide 664 against 604, 14336-wide 591
     // against 300, 11008-wide 640 either way)
-    if (iters > 32 && iters <= 44) return split_class(11, 4);
+    if (iters > 32 && iters <= 44) return split_class(11, 4) + (t.in_features % (4 * kWave) == 0 ? kExactClass : 0);
     if (iters > 16) return kLongClass;
     return 0;
 }
@@ -824,7 +869,8 @@ hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
 #undef MCC_CASE
         case kLongClass:
             return a.lr_scale != 0.0f ? launch_long_variant<true>(stream, a) : launch_long_variant<false>(stream, a);
-        case split_class(11, 4): return launch_split<11, 4>(stream, a);
+        case split_class(11, 4): return launch_split<11, 4, false>(stream, a);
+        case split_class(11, 4) + kExactClass: return launch_split<11, 4, true>(stream, a);
         default:
             return a.lr_scale != 0.0f ? launch_streamed_variant<true>(stream, a) : launch_streamed_variant<false>(stream, a);
     }

@@ -101,6 +101,23 @@ int main(int argc, char** argv) {
                 if ((int)got != exp) { if (mismatches < 10) std::printf("TABLE MISMATCH C=%d code=%d g=%d got=%u exp=%d\n", C, code, gi, got, exp); ++mismatches; }
             }
     }
+    // the reciprocal product tolerates a reciprocal that is off by a few units in the last place
+    // (the device refines the hardware's approximation instead of dividing)
+    for (long it = 0; it < 4000000; ++it) {
+        const float dn = log_uniform(1e-12, 1e12);
+        const float gw = (uni() < 0.5 ? -1.f : 1.f) * log_uniform(1e-18, 1e15);
+        double rd = 1.0 / (double)dn;
+        const int ulps = (int)(next_u64() % 9) - 4;
+        for (int u = 0; u < (ulps < 0 ? -ulps : ulps); ++u) rd = std::nextafter(rd, ulps < 0 ? 0.0 : 1e300);
+        if ((float)((double)gw * rd) != gw / dn) { std::printf("reciprocal product fails gw=%a dn=%a ulps=%d\n", gw, dn, ulps); return 2; }
+    }
+    // division by a power of two as a product with its reciprocal (finish_row_stats)
+    for (long it = 0; it < 2000000; ++it) {
+        const float x = (next_u64() & 7) ? log_uniform(1e-44, 1e38) : log_uniform(1e-45, 1e-36);
+        const int k = (int)(next_u64() % 21);
+        const mcc::RowStats a = mcc::finish_row_stats(x, 0.f, 0.f, 1.f, 1 << k, 0.f, 0.f, 0.f);
+        if (a.v_new != x / (float)(1 << k)) { std::printf("power-of-two division fails x=%a k=%d\n", x, k); return 2; }
+    }
     // collapsed seed xor: hash(seed ^ hash(elem)) == hash_rest(seed_mix(seed) ^ hash_open(hash_first(elem)))
     for (int i = 0; i < 4000000; ++i) {
         const uint32_t seed = (uint32_t)next_u64(), elem = (uint32_t)next_u64();
