@@ -23,9 +23,11 @@
 // rows whose four 16-byte chunks are XOR-swizzled with bits 2-3 of the row, which makes the
 // 16-byte MFMA operand reads (lane = row, 8 consecutive k) conflict-free without padding:
 // 32 or 40 KiB per workgroup.  Splitting and decoding are done by the thread that fetched the
-// data, on its way into LDS; per slab and thread that is about 200 VALU instructions against
-// 24 MFMAs, so the kernel runs near a third of the bf16 matrix peak -- twice the fp32 matrix
-// peak in algorithmic flops.
+// data, on its way into LDS.  The whole-tile kernel decodes through a table: two neighbouring
+// 6-bit codes of a packed word index a 4096-entry LDS table (16 KiB, built once per workgroup)
+// whose entries are their two ternary values as a bf16 pair, so a packed group costs two table
+// reads and four address instructions instead of 22 instructions of arithmetic -- the vector work
+// per slab, which competes with the matrix instructions for issue slots, drops by about a third.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -74,7 +76,11 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
     constexpr int kA4 = kT * kK / 4 / kThreads;  // float4 of activation per thread and slab
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * kPlaneBytes];
     __shared__ __attribute__((aligned(16))) uint8_t lds_b[kTN * kRowBytes];
+    // pair_t[c1 << 6 | c0] = bf16(t(c0)) | bf16(t(c1)) << 16 with t = code / lv - 1
+    __shared__ uint32_t pair_t[4096];
     const int tid = threadIdx.x;
+    for (int i = tid; i < 4096; i += kThreads)
+        pair_t[i] = pack_bf16((float)(code_q((uint32_t)i & 63u, a.cd) - 1), (float)(code_q((uint32_t)i >> 6, a.cd) - 1));
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, kh = lane >> 5;
     const int wm0 = (wave / WN) * 64, wn0 = (wave % WN) * 64;
@@ -143,23 +149,31 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
             rw[p] = w >> (8 * is_last);
         }
     };
-    auto ternary = [&](uint32_t word, int k) { return (float)(code_q(code_of(word, k), a.cd) - 1); };
+    // the ternary values of codes 0, 1 (low pair) and 2, 3 (high pair) of a packed word, as bf16 pairs
+    auto pair_lo = [&](uint32_t word) { return pair_t[word & 0xfffu]; };
+    auto pair_hi = [&](uint32_t word) { return pair_t[(word >> 12) & 0xfffu]; };
     auto stage = [&]() {
 #pragma unroll
         for (int p = 0; p < kA4; ++p) store_split(lds_a, lds_off_a[p], ra[p].x, ra[p].y, ra[p].z, ra[p].w);
         if (FORWARD) {
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const uint32_t lo = pack_bf16(ternary(rw[p], 0), ternary(rw[p], 1));
-                const uint32_t hi = pack_bf16(ternary(rw[p], 2), ternary(rw[p], 3));
-                *reinterpret_cast<uint2*>(lds_b + lds_off_b[p]) = make_uint2(lo, hi);
-            }
+            for (int p = 0; p < 4; ++p)
+                *reinterpret_cast<uint2*>(lds_b + lds_off_b[p]) = make_uint2(pair_lo(rw[p]), pair_hi(rw[p]));
         } else {
+            // rw[r] is weight row k = 4 oq + r; column 4 g + j takes code j of each: the pairs come
+            // out of the table along a row and are transposed two by two (v_perm_b32)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {  // rw[r] is weight row k = 4 oq + r; column 4 g + j takes code j of each
-                const uint32_t lo = pack_bf16(ternary(rw[0], j), ternary(rw[1], j));
-                const uint32_t hi = pack_bf16(ternary(rw[2], j), ternary(rw[3], j));
-                *reinterpret_cast<uint2*>(lds_b + lds_off_b[j]) = make_uint2(lo, hi);
+            for (int h = 0; h < 2; ++h) {  // codes 2 h, 2 h + 1
+                uint32_t pr[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) pr[r] = h == 0 ? pair_lo(rw[r]) : pair_hi(rw[r]);
+                // column 2 h: the low halves of rows (0, 1) and (2, 3); column 2 h + 1: the high halves
+                const uint32_t lo0 = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u);
+                const uint32_t hi0 = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u);
+                const uint32_t lo1 = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);
+                const uint32_t hi1 = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
+                *reinterpret_cast<uint2*>(lds_b + lds_off_b[2 * h]) = make_uint2(lo0, hi0);
+                *reinterpret_cast<uint2*>(lds_b + lds_off_b[2 * h + 1]) = make_uint2(lo1, hi1);
             }
         }
     };
@@ -172,6 +186,7 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
 
     uint32_t w_base = 0;
     fetch(0, 0);
+    __syncthreads();  // the table is complete
     for (int k0 = 0; k0 < K; k0 += kK) {
         stage();
         __syncthreads();
