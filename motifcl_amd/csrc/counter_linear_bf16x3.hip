@@ -31,6 +31,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 #include "bf16_split.hpp"
 #include "counter_math.hpp"
@@ -228,6 +229,272 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
         }
 }
 
+// The same tile (128 rows x 256 columns) with the two kinds of work on different waves: one
+// workgroup of 16 waves per CU, of which waves 0-7 only multiply (32 rows x 128 columns each: per
+// slab 24 matrix instructions and 14 operand reads) and waves 8-15 only stage (the slab between
+// them: 8 activations and 4 packed groups per thread), two of each kind on every SIMD.  In the
+// kernel above every wave stages and then multiplies, the waves of a SIMD do so in step, and the
+// matrix pipe idles while they stage (busy 54 % of the cycles); here the SIMD's matrix pipe and
+// its vector ALUs work at the same time on different waves (68 %).  Two LDS buffers (the stagers
+// fill one while the other is multiplied), one barrier per slab.  What made the difference, in
+// the order found:
+//   - nothing computed from a loaded value inside the fetch (it would wait for the load there),
+//     and a steady-state loop without conditions (the compiler's wait counts are the minimum over
+//     all paths into a point: one path with fewer loads in flight and every wait drains them), so
+//     the stagers' loads stay three to four slabs ahead;
+//   - the multiplying waves read the operands of a 16-deep step while the matrix instructions of
+//     the step before run (two register sets), and the slab's barrier sits between its two steps;
+//   - 32 x 128 wave tiles: 7 operand reads per 12 matrix instructions where 64 x 64 needs 8 (the
+//     activation has three planes, so a wave tile should be wide, not tall); LDS instruction
+//     count is what the two kinds of wave compete for;
+//   - the last-group handling (a byte early, shifted) only in the slabs that can hold that group.
+template <bool FORWARD>
+__global__ __launch_bounds__(1024, 4) void counter_linear_bf16x3_split_roles_kernel(Lin3Args a) {
+    constexpr int CW = 8;  // multiplying waves; as many staging waves
+    constexpr int kTN = 256;
+    constexpr int kStagers = 64 * CW;                  // threads of the staging waves
+    constexpr int kA4 = kT * kK / 4 / kStagers;        // 2 float4 of activation per stager and slab
+    constexpr int kW = kTN * kK / 4 / kStagers;        // 4 packed groups per stager and slab
+    constexpr int kBufA = 3 * kPlaneBytes, kBufB = kTN * kRowBytes;
+    // One array, the table first: its entries are then addressed by their byte offset alone.
+    // pair_t[c1 << 6 | c0] = bf16(t(c0)) | bf16(t(c1)) << 16 with t = code / lv - 1
+    constexpr int kTableBytes = 4096 * 4;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kTableBytes + 2 * kBufA + 2 * kBufB];
+    uint32_t* pair_t = reinterpret_cast<uint32_t*>(lds);
+    auto lds_a = [&](int buf) { return lds + kTableBytes + buf * kBufA; };
+    auto lds_b = [&](int buf) { return lds + kTableBytes + 2 * kBufA + buf * kBufB; };
+    const int tid = threadIdx.x;
+    for (int i = tid; i < 4096; i += 128 * CW)
+        pair_t[i] = pack_bf16((float)(code_q((uint32_t)i & 63u, a.cd) - 1), (float)(code_q((uint32_t)i >> 6, a.cd) - 1));
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool stager = wave >= CW;  // wave-uniform
+    const TileXY tile = xcd_tile(gridDim.x, gridDim.y, 4);
+    const int m0 = tile.y * kT, n0 = tile.x * kTN;
+    const int K = FORWARD ? a.in_features : a.out_features;
+    const int N = FORWARD ? a.out_features : a.in_features;
+    const int slabs = K / kK;
+
+    if (stager) {
+        constexpr int kRows = kStagers / 8;  // rows of 8 groups one pass of the stagers covers
+        const int st = tid - kStagers;
+        const int c4 = st & 7, row0 = st >> 3;  // row0 in [0, kRows)
+        const uint32_t gpr = (uint32_t)a.in_features >> 2;
+        const uint32_t last_off = 3u * ((uint32_t)a.out_features * gpr - 1u);
+        uint32_t off_a[kA4], off_w[kW];
+        int lds_off_a[kA4], lds_off_b[kW];
+#pragma unroll
+        for (int p = 0; p < kA4; ++p) {
+            const int row = row0 + kRows * p;
+            off_a[p] = ((uint32_t)(m0 + row) * (uint32_t)K + 4u * c4) * 4u;
+            lds_off_a[p] = tile_offset(row, c4 >> 1, c4 & 1);
+        }
+#pragma unroll
+        for (int p = 0; p < kW; ++p) {
+            if (FORWARD) {
+                // (weight row n = row0 + kRows p, group c4 of the slab)
+                const int n = row0 + kRows * p;
+                off_w[p] = 3u * ((uint32_t)(n0 + n) * gpr + (uint32_t)c4);
+                lds_off_b[p] = tile_offset(n, c4 >> 1, c4 & 1);
+            } else {
+                // p = 4 q + r: weight row k = 4 oq + r (oq = c4), group g = row0 + kRows q of the tile's columns;
+                // after the transpose, slot 4 q + j holds column 4 g + j
+                const int q = p >> 2, r = p & 3, g = row0 + kRows * q;
+                off_w[p] = 3u * ((uint32_t)(4 * c4 + r) * gpr + (uint32_t)(n0 >> 2) + (uint32_t)g);
+                lds_off_b[p] = dealt_tile_offset<kTN>(4 * g + r, c4 >> 1, c4 & 1);
+            }
+        }
+        const uint32_t w_step = FORWARD ? 3u * (kK / 4) : 3u * kK * gpr;  // packed bytes per slab
+        // What a fetch leaves in registers is exactly what the loads return: anything computed from it
+        // here would wait for the load at once instead of kAhead slabs later.
+        struct Fetched {
+            float4 ra[kA4];
+            float4 sc;
+            uint32_t rw[kW];
+        };
+        // Only the tensor's last packed group has no byte after it, and it lies in the last slab: the
+        // careful forms (which fetch it one byte early and shift) are used for the last slabs only.
+        using Careful = std::true_type;
+        using Plain = std::false_type;
+        auto fetch = [&](auto careful, int slab, Fetched& f) {
+            const int k0 = slab * kK;
+            const uint32_t w_base = (uint32_t)slab * w_step;
+            if (!FORWARD) f.sc = *reinterpret_cast<const float4*>(a.scale + k0 + 4 * c4);
+#pragma unroll
+            for (int p = 0; p < kA4; ++p)
+                f.ra[p] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.act) + off_a[p] +
+                                                           4u * (uint32_t)k0);
+#pragma unroll
+            for (int p = 0; p < kW; ++p) {
+                uint32_t off = off_w[p] + w_base;  // one 4-byte load per packed group
+                if constexpr (decltype(careful)::value) off -= off == last_off ? 1u : 0u;
+                __builtin_memcpy(&f.rw[p], a.state + off, 4);
+            }
+        };
+        auto pair_lo = [&](uint32_t word) { return *reinterpret_cast<const uint32_t*>(lds + ((word << 2) & 0x3ffcu)); };
+        auto pair_hi = [&](uint32_t word) { return *reinterpret_cast<const uint32_t*>(lds + ((word >> 10) & 0x3ffcu)); };
+        auto stage = [&](auto careful, int buf, int slab, const Fetched& f) {
+            uint8_t* pa = lds_a(buf);
+            uint8_t* pb = lds_b(buf);
+            uint32_t rw[kW];
+#pragma unroll
+            for (int p = 0; p < kW; ++p) {
+                rw[p] = f.rw[p];
+                if constexpr (decltype(careful)::value)
+                    rw[p] >>= off_w[p] + (uint32_t)slab * w_step == last_off ? 8 : 0;
+            }
+            // all table reads first (their latency passes under the split of the activations), then the
+            // writes: both are in the one LDS array, and a read after a write would wait for it
+            uint32_t lo[kW], hi[kW];
+#pragma unroll
+            for (int p = 0; p < kW; ++p) {
+                lo[p] = pair_lo(rw[p]);
+                hi[p] = pair_hi(rw[p]);
+            }
+#pragma unroll
+            for (int p = 0; p < kA4; ++p) {
+                float4 x = f.ra[p];
+                // (grad_out * scale) first, as the reference does
+                if (!FORWARD) x = make_float4(x.x * f.sc.x, x.y * f.sc.y, x.z * f.sc.z, x.w * f.sc.w);
+                store_split(pa, lds_off_a[p], x.x, x.y, x.z, x.w);
+            }
+            if (FORWARD) {
+#pragma unroll
+                for (int p = 0; p < kW; ++p) *reinterpret_cast<uint2*>(pb + lds_off_b[p]) = make_uint2(lo[p], hi[p]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < kW / 4; ++q)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {  // codes 2 h, 2 h + 1 of rows k .. k + 3
+                        uint32_t pr[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) pr[r] = h == 0 ? lo[4 * q + r] : hi[4 * q + r];
+                        const uint32_t lo0 = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u);
+                        const uint32_t hi0 = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u);
+                        const uint32_t lo1 = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);
+                        const uint32_t hi1 = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
+                        *reinterpret_cast<uint2*>(pb + lds_off_b[4 * q + 2 * h]) = make_uint2(lo0, hi0);
+                        *reinterpret_cast<uint2*>(pb + lds_off_b[4 * q + 2 * h + 1]) = make_uint2(lo1, hi1);
+                    }
+            }
+        };
+        // Slabs are fetched kAhead ahead of the one being staged (kAhead register sets), so a load has
+        // that many slab times to arrive.
+        constexpr int kAhead = FORWARD ? 4 : 3;
+        Fetched f[kAhead];
+#pragma unroll
+        for (int d = 0; d < kAhead; ++d) fetch(Plain{}, d, f[d]);
+        __syncthreads();  // the table is complete
+        stage(Plain{}, 0, 0, f[0]);
+        fetch(Plain{}, kAhead, f[0]);  // slabs > 2 kAhead + 1 (the launcher's condition)
+        __syncthreads();               // slab 0 is in buffer 0
+        // The steady state has no conditions: every path through it has the same loads in flight, so
+        // the compiler's wait counts let the newest kAhead - 1 sets stay in flight.  It stops short
+        // of fetching the last slab.
+        int s = 0;
+        for (; s + 2 * kAhead + 1 < slabs; s += kAhead) {
+#pragma unroll
+            for (int d = 0; d < kAhead; ++d) {
+                // while the other waves multiply slab s + d: slab s + d + 1 into the other buffer
+                const int nxt = (d + 1) % kAhead;
+                stage(Plain{}, (s + d + 1) & 1, s + d + 1, f[nxt]);
+                fetch(Plain{}, s + d + 1 + kAhead, f[nxt]);
+                __syncthreads();
+            }
+        }
+        for (; s < slabs; s += kAhead) {
+#pragma unroll
+            for (int d = 0; d < kAhead; ++d) {
+                if (s + d >= slabs) break;
+                const int nxt = (d + 1) % kAhead;
+                if (s + d + 1 < slabs) stage(Careful{}, (s + d + 1) & 1, s + d + 1, f[nxt]);
+                if (s + d + 1 + kAhead < slabs) fetch(Careful{}, s + d + 1 + kAhead, f[nxt]);
+                __syncthreads();
+            }
+        }
+        return;
+    }
+
+    // The multiplying waves, 32 rows x 128 columns each.  A slab is two 16-deep steps; the operands
+    // of a step (3 activation reads, 4 weight reads) are read into registers while the matrix
+    // instructions of the step before run, so no read's latency is waited for.  The slab's barrier
+    // sits between its two steps: by then this wave has read all of the slab (the stagers may
+    // overwrite it) and the stagers have finished the next slab (its first step's operands are read
+    // during this slab's second step).
+    const int l32 = lane & 31, kh = lane >> 5;
+    constexpr int kAcross = 2;                 // multiplying waves side by side
+    constexpr int kWaveN = kTN / kAcross;      // columns per wave
+    constexpr int kWaveM = kT / (CW / kAcross);  // rows per wave
+    constexpr int IB = kWaveM / 32, JB = kWaveN / 32;
+    constexpr int kReads = 3 * IB + JB, kMfma = 3 * IB * JB;
+    const int wm0 = kWaveM * (wave / kAcross), wn0 = kWaveN * (wave % kAcross);
+    floatx16 acc[IB][JB];
+#pragma unroll
+    for (int i = 0; i < IB; ++i)
+#pragma unroll
+        for (int j = 0; j < JB; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    auto read_step = [&](int buf, int c, bf16x8 (&fa)[3][IB], bf16x8 (&fb)[JB]) {
+        const uint8_t* pa = lds_a(buf);
+        const uint8_t* pb = lds_b(buf);
+        const int chunk = 2 * c + kh;  // lane half kh holds k = 8 chunk .. 8 chunk + 7
+#pragma unroll
+        for (int j = 0; j < JB; ++j)
+            fb[j] = FORWARD ? read_operand(pb, wn0 + 32 * j + l32, chunk)
+                            : read_dealt_operand<kTN>(pb, wn0 + 32 * j + l32, chunk);
+#pragma unroll
+        for (int plane = 0; plane < 3; ++plane)
+#pragma unroll
+            for (int i = 0; i < IB; ++i) fa[plane][i] = read_operand(pa + plane * kPlaneBytes, wm0 + 32 * i + l32, chunk);
+    };
+    auto multiply_step = [&](const bf16x8 (&fa)[3][IB], const bf16x8 (&fb)[JB]) {
+#pragma unroll
+        for (int plane = 0; plane < 3; ++plane)
+#pragma unroll
+            for (int i = 0; i < IB; ++i)
+#pragma unroll
+                for (int j = 0; j < JB; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[plane][i], fb[j], acc[i][j], 0, 0, 0);
+    };
+    // the matrix instructions of a step with the operand reads of the next step between the first of
+    // them, so the reads have landed when the step ends
+    auto interleave = [&]() {
+#pragma unroll
+        for (int g = 0; g < kReads; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // matrix
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kReads, 0);
+    };
+    bf16x8 fa0[3][IB], fb0[JB], fa1[3][IB], fb1[JB];
+    __syncthreads();  // the table is complete (the stagers' barrier)
+    __syncthreads();  // slab 0 is in buffer 0
+    read_step(0, 0, fa0, fb0);
+    for (int s = 0; s < slabs; ++s) {
+        read_step(s & 1, 1, fa1, fb1);
+        multiply_step(fa0, fb0);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);  // all of the step before the barrier: its last reads land meanwhile
+        __syncthreads();
+        read_step((s + 1) & 1, 0, fa0, fb0);  // after the last slab: read and never used
+        multiply_step(fa1, fb1);
+        interleave();
+    }
+#pragma unroll
+    for (int i = 0; i < IB; ++i)
+#pragma unroll
+        for (int j = 0; j < JB; ++j) {
+            const int col = n0 + wn0 + 32 * j + l32;
+            const float sv = FORWARD ? a.scale[col] : 1.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm0 + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+                a.c[(size_t)row * N + col] = FORWARD ? acc[i][j][r] * sv : acc[i][j][r];
+            }
+        }
+}
+
 // Any shape: every access is checked and short slabs are zero-filled.
 template <bool FORWARD, bool VEC_A>
 __global__ __launch_bounds__(kGemmThreads, 3) void counter_linear_bf16x3_edge_kernel(Lin3Args a) {
@@ -376,8 +643,13 @@ hipError_t launch_lin3(hipStream_t stream, const float* act, const uint8_t* stat
     // 256-column tiles (8 waves) share one split of the activation slab between twice as many
     // columns: +15 % when there are enough of them to fill the device
     if (whole && N % 256 == 0 && (long)(rows / kT) * (N / 256) >= 256) {
-        hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 4>), dim3(N / 256, rows / kT), dim3(512), 0, stream,
-                           a);
+        // 16 slabs or more: the staging waves run four slabs ahead
+        if (K >= 16 * kK)
+            hipLaunchKernelGGL((counter_linear_bf16x3_split_roles_kernel<FORWARD>), dim3(N / 256, rows / kT), dim3(1024),
+                               0, stream, a);
+        else
+            hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 4>), dim3(N / 256, rows / kT), dim3(512), 0, stream,
+                               a);
         return hipGetLastError();
     }
     const dim3 grid((N + kT - 1) / kT, (rows + kT - 1) / kT);

@@ -8,6 +8,9 @@ together) meet the oracle the same way at 16384 tokens -- half the config's toke
 halves the oracle's 22 s per case and takes the same kernels -- through the full workspace, and
 the strip workspace (parked tiles, no gradient buffer) must give the full workspace's bytes.
 cfg3: one tensor of each shape of the 224 at full size, update-only, bit-exact.
+Forward and grad_x of the layer's three shapes at the full 32768 tokens: 96 sampled rows (every
+128-row tile band has the same code path; the sample always holds the first and the last row)
+against a double-precision product with the oracle's decoded weight.
 The oracle needs a few seconds per case on 16 threads."""
 import numpy as np
 import pytest
@@ -103,3 +106,28 @@ def test_cfg3_tensor_update_only_is_bit_exact(ops, oracle, shape):
     for a, b in zip([t.cpu().numpy() for t in st], exp):
         assert np.array_equal(a, b)
     assert float((oracle.unpack_codes(exp[0]) != oracle.unpack_codes(h0[0])).mean()) > 0.5  # the step did something
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (11008, 4096), (4096, 11008)], ids=lambda s: "%dx%d" % s)
+def test_cfg4_forward_and_grad_x_at_32768_tokens_on_sampled_rows(ops, oracle, shape):
+    tokens = 32768
+    n_out, n_in = shape
+    x = ops.fill_normal(torch.empty(tokens, n_in, device="cuda"), 301, 1.0)
+    dy = ops.fill_normal(torch.empty(tokens, n_out, device="cuda"), 302, 0.01)
+    state, scale, _ = make_state(ops, n_out, n_in, 303)
+    # per-row scales that differ, so a scale applied to the wrong row or column shows
+    scale.mul_(torch.linspace(0.5, 1.5, n_out, device="cuda"))
+    y = ops.forward(x, state, scale, C, n_out)
+    gx = ops.backward_input(dy, state, scale, C, n_in)
+    torch.cuda.synchronize()
+    rows = np.unique(np.concatenate([[0, tokens - 1], np.random.default_rng(7).integers(0, tokens, 94)]))
+    idx = torch.from_numpy(rows).cuda()
+    w = oracle.decode_weight(state.cpu().numpy(), scale.cpu().numpy(), C, n_in, n_out).astype(np.float64)
+    y_ref = x[idx].cpu().numpy().astype(np.float64) @ w.T
+    gx_ref = dy[idx].cpu().numpy().astype(np.float64) @ w
+    e_y = np.abs(y[idx].cpu().numpy() - y_ref).max() / np.abs(y_ref).max()
+    e_gx = np.abs(gx[idx].cpu().numpy() - gx_ref).max() / np.abs(gx_ref).max()
+    print("cfg4 [%d,%d]@%d: forward max err / max|y| = %.2e, grad_x %.2e" % (n_out, n_in, tokens, e_y, e_gx))
+    # tests/test_vulkan_counter_fused.cpp:107 allows 2e-5; exactly split activations give the accuracy of an
+    # fp32 sum (about 1.5e-6 at these lengths)
+    assert e_y <= 4e-6 and e_gx <= 4e-6
