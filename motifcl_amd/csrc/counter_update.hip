@@ -605,12 +605,12 @@ struct SplitShared {
     int fast_div;
 };
 
-constexpr int min_waves_split(int j) { return j <= 6 ? 4 : 3; }
+constexpr int min_waves_split(int j) { return j <= 6 ? 4 : j <= 11 ? 3 : 2; }
 
 // ALIGNED: rows of a whole number of 256-weight iterations (11008 = 43 * 256): no lane is ever
 // masked, an iteration past the row's end is skipped by the whole wave, and every iteration is an
 // aligned span of the element index, so the first hash products come by addition (hash_delta).
-template <int J, int W, bool WITH_GS, bool ALIGNED>
+template <int J, int W, bool WITH_GS, bool ALIGNED, bool EVEN>
 __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_split_kernel(BatchArgs a) {
     __shared__ SplitShared sh;
     const int lane = threadIdx.x & (kWave - 1);
@@ -620,12 +620,18 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
     const bool last_row = row == t.out_features - 1;
     const uint32_t gpr = (uint32_t)t.in_features >> 2;
     const int iters = (int)((gpr + kWave - 1) / kWave);
-    const int j0 = w * J;
+    // the row's iterations in W stretches: of J (EVEN false: the class of one row length, whose
+    // stretches of J are even already and whose loops then carry no second bound), or of jn <= J,
+    // as even as the row's length allows
+    const int jn = EVEN ? (iters + W - 1) / W : J;
+    const int j0 = w * jn;
     const float4* g_row = reinterpret_cast<const float4*>(t.grad_w + (size_t)row * t.in_features);
     uint8_t* s_row = t.state + (size_t)row * gpr * 3;
+    // whether iteration j0 + jj is this wave's and inside the row (wave-uniform)
+    auto mine = [&](int jj) { return (!EVEN || jj < jn) && j0 + jj < iters; };
     // whether lane's group of iteration j0 + jj exists: per iteration when ALIGNED
     auto live_at = [&](int jj) {
-        return ALIGNED ? j0 + jj < iters : (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr;
+        return mine(jj) && (ALIGNED || (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj) < gpr);
     };
 
     float4 q[J];
@@ -633,20 +639,15 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
 #pragma unroll
     for (int jj = 0; jj < J; ++jj) {
         const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
-        if (ALIGNED) {
-            if (j0 + jj < iters) {  // wave-uniform
-                q[jj] = load_grad4_once(g_row + gi);
-                words[jj] = last_row ? load_group_dword_or_tail_once(s_row + 3u * gi, gi == gpr - 1)
-                                     : load_group_dword_once(s_row + 3u * gi);
-            } else {
-                q[jj] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                words[jj] = 0u;
-            }
-        } else {
-            const uint32_t gc = gi < gpr ? gi : gpr - 1;
+        if (mine(jj)) {
+            // lanes past the end of a ragged row re-read its last group and are masked below
+            const uint32_t gc = ALIGNED || gi < gpr ? gi : gpr - 1;
             q[jj] = load_grad4_once(g_row + gc);
             words[jj] = last_row ? load_group_dword_or_tail_once(s_row + 3u * gc, gc == gpr - 1)
                                  : load_group_dword_once(s_row + 3u * gc);
+        } else {
+            q[jj] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            words[jj] = 0u;
         }
     }
     build_luts(sh.luts, a.cd, a.geom);  // while the row is in flight
@@ -661,7 +662,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
 #pragma unroll
         for (int jj = 0; jj < J; ++jj) {
             // a skipped iteration holds zeros: +0.0 to the sums, the largest key to the minimum
-            const bool live = ALIGNED || live_at(jj);
+            const bool live = ALIGNED || live_at(jj);  // (a skipped iteration of a whole row holds zeros already)
             const float g[4] = {live ? q[jj].x : 0.0f, live ? q[jj].y : 0.0f, live ? q[jj].z : 0.0f,
                                 live ? q[jj].w : 0.0f};
             my_key = umin3(my_key, range_key(g[0]), range_key(g[1]));
@@ -720,7 +721,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
     asm volatile("" : "+v"(rc.tc.neg_lr), "+v"(rc.tc.k), "+v"(rc.tc.two_m24), "+v"(rc.tc.seed_mix));  // VGPR operands
     const bool fast = __builtin_amdgcn_readfirstlane(sh.fast_div) != 0;
     if (!fast || (!WITH_GS && !scale_unchanged(rc))) {
-        apply_streamed(t, row, lane, rc, sh.luts, j0 * kWave, (j0 + J) * kWave);
+        apply_streamed(t, row, lane, rc, sh.luts, j0 * kWave, (j0 + jn) * kWave);
         return;
     }
     const RebasedCounters rebased{sh.luts.c_f, WITH_GS ? rebase_ratio(rc) : 1.0f};
@@ -729,7 +730,7 @@ __global__ __launch_bounds__(kWave* W, min_waves_split(J)) void update_rows_spli
     uint32_t dv_bits = 4u;
 #pragma unroll
     for (int jj = 0; jj < J; ++jj) {
-        if (j0 + jj < iters) {  // wave-uniform
+        if (mine(jj)) {
             const uint32_t gi = (uint32_t)lane + (uint32_t)kWave * (uint32_t)(j0 + jj);
             const float g[4] = {q[jj].x, q[jj].y, q[jj].z, q[jj].w};
             uint32_t nw;
@@ -791,7 +792,8 @@ hipError_t launch_streamed_variant(hipStream_t stream, const BatchArgs& a) {
 template <int J, int W, bool WITH_GS, bool ALIGNED>
 hipError_t launch_split_variant(hipStream_t stream, const BatchArgs& a) {
     const dim3 grid((unsigned)a.t[0].out_features, (unsigned)a.n_tensors);
-    hipLaunchKernelGGL((update_rows_split_kernel<J, W, WITH_GS, ALIGNED>), grid, dim3(kWave * W), 0, stream, a);
+    // 11008-wide rows (43 iterations) fall into four stretches of 11 as they are
+    hipLaunchKernelGGL((update_rows_split_kernel<J, W, WITH_GS, ALIGNED, J != 11>), grid, dim3(kWave * W), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -824,8 +826,9 @@ hipError_t launch_iters(hipStream_t stream, const BatchArgs& a) {
 }
 
 // Row lengths (in units of 64 groups = 256 weights, rounded up) with a one-wave
-// register-resident variant: every length up to 4096 weights.  Longer rows are read twice by
-// one wave, except 8192 < length <= 11264, which four waves share register-resident.
+// register-resident variant: every length up to 4096 weights.  Longer rows, up to 32768 weights,
+// are shared register-resident by 4, 8 or 16 cooperating waves; beyond that one wave reads the
+// row twice.
 #define MCC_RESIDENT_ITERS(X) \
     X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16)
 
@@ -847,11 +850,15 @@ int iters_class(const UpdateTensor& t) {
         return iters + (t.in_features == 4 * kWave * iters ? kExactClass : 0);
         default: break;
     }
-    // 11008-wide rows (the 7B FFN width) stay with four cooperating waves, which read the row
-    // once; every other long row takes the two-pass wave (measured at 4096 rows: 5120-wide 639
-    // against 425 Gweights/s for the cooperating waves, 8192-wide 664 against 604, 14336-wide 591
-    // against 300, 11008-wide 640 either way)
-    if (iters > 32 && iters <= 44) return split_class(11, 4) + (t.in_features % (4 * kWave) == 0 ? kExactClass : 0);
+    // Cooperating waves, one row per workgroup, each wave a stretch of at most 8 iterations (11 for
+    // the 7B FFN width): 4 waves up to 8192 weights, 8 up to 16384, 16 up to 32768.  Measured at
+    // 4096 rows against the two-pass wave: 5120-wide 0.60 against 0.48 of the HBM peak, 8192-wide
+    // 0.66 / 0.49, 14336-wide 0.58 / 0.46, 28672-wide 0.44 / 0.37, 20480-wide 0.40 either way.
+    const int exact = t.in_features % (4 * kWave) == 0 ? kExactClass : 0;
+    if (iters <= 32) return split_class(8, 4) + exact;
+    if (iters <= 44) return split_class(11, 4) + exact;
+    if (iters <= 64) return split_class(8, 8) + exact;
+    if (iters <= 128) return split_class(8, 16) + exact;
     if (iters > 16) return kLongClass;
     return 0;
 }
@@ -869,8 +876,14 @@ hipError_t launch_class(hipStream_t stream, int cls, const BatchArgs& a) {
 #undef MCC_CASE
         case kLongClass:
             return a.lr_scale != 0.0f ? launch_long_variant<true>(stream, a) : launch_long_variant<false>(stream, a);
-        case split_class(11, 4): return launch_split<11, 4, false>(stream, a);
-        case split_class(11, 4) + kExactClass: return launch_split<11, 4, true>(stream, a);
+#define MCC_SPLIT_CASE(J, W)                                               \
+    case split_class(J, W): return launch_split<J, W, false>(stream, a); \
+    case split_class(J, W) + kExactClass: return launch_split<J, W, true>(stream, a);
+        MCC_SPLIT_CASE(8, 4)
+        MCC_SPLIT_CASE(11, 4)
+        MCC_SPLIT_CASE(8, 8)
+        MCC_SPLIT_CASE(8, 16)
+#undef MCC_SPLIT_CASE
         default:
             return a.lr_scale != 0.0f ? launch_streamed_variant<true>(stream, a) : launch_streamed_variant<false>(stream, a);
     }

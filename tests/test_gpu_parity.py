@@ -44,8 +44,11 @@ DENSE_SHAPES = [
     (288, 288, 11), (768, 288, 11), (288, 768, 11), (96, 2048, 11), (48, 4096, 11),
     (12, 11008, 11), (5, 260, 11), (7, 1028, 8), (3, 3076, 11), (5, 6144, 11),
     (3, 8192, 4), (2, 11012, 11), (3, 16384, 11), (9, 516, 1),
-    # long rows read twice by one wave: below and above the 11008-wide class, chunk tails, very long
+    # long rows shared by four or eight cooperating waves in equal stretches: whole and ragged rows in
+    # every class (up to 8192, 11264, 16384, 32768 weights), uneven last stretches, and beyond them
+    # the rows one wave reads twice
     (4, 4352, 11), (3, 8448, 11), (3, 11268, 11), (2, 28672, 11), (2, 22532, 3),
+    (3, 4100, 11), (2, 5120, 11), (2, 13824, 11), (2, 14336, 4), (2, 32768, 11), (2, 32772, 3), (1, 40960, 11),
 ]
 
 
