@@ -636,30 +636,57 @@ hipError_t launch_lin3(hipStream_t stream, const float* act, const uint8_t* stat
     const int N = FORWARD ? out_features : in_features;
     const int K = FORWARD ? in_features : out_features;
     const bool vec_a = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(act) & 15u) == 0);
-    const bool whole = rows % kT == 0 && N % kT == 0 && K % kK == 0 && vec_a &&
-                       (reinterpret_cast<uintptr_t>(scale) & 15u) == 0 &&
-                       (uint64_t)rows * (uint64_t)K * 4u < (1ull << 32) &&
-                       (uint64_t)out_features * (uint64_t)in_features * 3u / 4u < (1ull << 32);
-    // 256-column tiles (8 waves) share one split of the activation slab between twice as many
-    // columns: +15 % when there are enough of them to fill the device
-    if (whole && N % 256 == 0 && (long)(rows / kT) * (N / 256) >= 256) {
-        // 16 slabs or more: the staging waves run four slabs ahead
-        if (K >= 16 * kK)
-            hipLaunchKernelGGL((counter_linear_bf16x3_split_roles_kernel<FORWARD>), dim3(N / 256, rows / kT), dim3(1024),
-                               0, stream, a);
+    const dim3 edge_block(kGemmThreads);
+    auto launch_edge = [&](const Lin3Args& e) {
+        const dim3 grid((N + kT - 1) / kT, (e.rows + kT - 1) / kT);
+        if (vec_a)
+            hipLaunchKernelGGL((counter_linear_bf16x3_edge_kernel<FORWARD, true>), grid, edge_block, 0, stream, e);
         else
-            hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 4>), dim3(N / 256, rows / kT), dim3(512), 0, stream,
-                               a);
+            hipLaunchKernelGGL((counter_linear_bf16x3_edge_kernel<FORWARD, false>), grid, edge_block, 0, stream, e);
         return hipGetLastError();
+    };
+    // whole 128-column tiles and whole slabs, aligned operands, a packed weight below 4 GiB
+    const bool shape_whole = N % kT == 0 && K % kK == 0 && vec_a && (reinterpret_cast<uintptr_t>(scale) & 15u) == 0 &&
+                             (uint64_t)out_features * (uint64_t)in_features * 3u / 4u < (1ull << 32);
+    if (!shape_whole || rows < kT) return launch_edge(a);
+    // The unchecked kernels take whole 128-row tiles and address the activations with 32-bit byte
+    // offsets: the rows go out in launches of whole tiles below 4 GiB of activations each, and a
+    // ragged rest of fewer than 128 rows goes to the checked kernel.
+    // (and the grid's y extent is at most 65535 tiles)
+    const uint64_t fit_rows = ((1ull << 32) - 1) / ((uint64_t)K * 4u) / kT * kT;
+    const int max_rows = (int)(fit_rows < 65535ull * kT ? fit_rows : 65535ull * kT);
+    const int whole_rows = rows / kT * kT;
+    if (max_rows < kT) return launch_edge(a);
+    for (int r0 = 0; r0 < whole_rows; r0 += max_rows) {
+        Lin3Args w = a;
+        w.rows = whole_rows - r0 < max_rows ? whole_rows - r0 : max_rows;
+        w.act = act + (size_t)r0 * K;
+        w.c = c + (size_t)r0 * N;
+        // 256-column tiles share one split of the activation slab between twice as many columns:
+        // +15 % when there are enough of them to fill the device
+        if (N % 256 == 0 && (long)(w.rows / kT) * (N / 256) >= 256) {
+            // 16 slabs or more: the staging waves run four slabs ahead
+            if (K >= 16 * kK)
+                hipLaunchKernelGGL((counter_linear_bf16x3_split_roles_kernel<FORWARD>), dim3(N / 256, w.rows / kT),
+                                   dim3(1024), 0, stream, w);
+            else
+                hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 4>), dim3(N / 256, w.rows / kT), dim3(512), 0,
+                                   stream, w);
+        } else {
+            hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 2>), dim3(N / kT, w.rows / kT), dim3(kGemmThreads), 0,
+                               stream, w);
+        }
+        const hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return err;
     }
-    const dim3 grid((N + kT - 1) / kT, (rows + kT - 1) / kT);
-    if (whole)
-        hipLaunchKernelGGL((counter_linear_bf16x3_kernel<FORWARD, 2>), grid, dim3(kGemmThreads), 0, stream, a);
-    else if (vec_a)
-        hipLaunchKernelGGL((counter_linear_bf16x3_edge_kernel<FORWARD, true>), grid, dim3(kGemmThreads), 0, stream, a);
-    else
-        hipLaunchKernelGGL((counter_linear_bf16x3_edge_kernel<FORWARD, false>), grid, dim3(kGemmThreads), 0, stream, a);
-    return hipGetLastError();
+    if (rows > whole_rows) {
+        Lin3Args e = a;
+        e.rows = rows - whole_rows;
+        e.act = act + (size_t)whole_rows * K;
+        e.c = c + (size_t)whole_rows * N;
+        return launch_edge(e);
+    }
+    return hipSuccess;
 }
 
 }  // namespace

@@ -131,3 +131,29 @@ def test_cfg4_forward_and_grad_x_at_32768_tokens_on_sampled_rows(ops, oracle, sh
     # tests/test_vulkan_counter_fused.cpp:107 allows 2e-5; exactly split activations give the accuracy of an
     # fp32 sum (about 1.5e-6 at these lengths)
     assert e_y <= 4e-6 and e_gx <= 4e-6
+
+
+def test_forward_and_grad_x_beyond_4_gib_of_activations_with_a_ragged_end(ops, oracle):
+    # The unchecked kernels address the activations with 32-bit byte offsets and take whole 128-row
+    # tiles: 262216 rows x 4096 floats (4.3 GB) go out as one launch of 262016 rows, one of 128 rows
+    # and a checked launch of the last 72.  Rows on both sides of every seam against float64.
+    rows, wide, narrow = 262144 + 72, 4096, 256
+    seam = (2 ** 32 - 1) // (wide * 4) // 128 * 128
+    sample = np.array([0, 1, seam - 1, seam, seam + 127, seam + 128, rows - 73, rows - 72, rows - 1])
+    idx = torch.from_numpy(sample).cuda()
+    for name in ("forward", "grad_x"):
+        n_out, n_in = (narrow, wide) if name == "forward" else (wide, narrow)
+        act = ops.fill_normal(torch.empty(rows, wide, device="cuda"), 401, 1.0)
+        state, scale, _ = make_state(ops, n_out, n_in, 402)
+        scale.mul_(torch.linspace(0.5, 1.5, n_out, device="cuda"))
+        got = ops.forward(act, state, scale, C, n_out) if name == "forward" else ops.backward_input(act, state, scale, C, n_in)
+        torch.cuda.synchronize()
+        w = oracle.decode_weight(state.cpu().numpy(), scale.cpu().numpy(), C, n_in, n_out).astype(np.float64)
+        a = act[idx].cpu().numpy().astype(np.float64)
+        ref = a @ w.T if name == "forward" else a @ w
+        err = np.abs(got[idx].cpu().numpy() - ref).max() / np.abs(ref).max()
+        print("%s, %d rows x %d: max err / max|.| = %.2e on the seams" % (name, rows, wide, err))
+        assert err <= 4e-6
+        # nothing was left unwritten between the launches
+        assert bool(torch.isfinite(got).all()) and float(got.abs().sum(dim=1).min()) > 0.0
+        del act, got

@@ -303,7 +303,9 @@ LINEAR_SHAPES = [(2, 4, 2, 3), (37, 68, 35, 3), (64, 256, 256, 11), (100, 288, 7
                  # 256 such tiles and 16 slabs or more: the kernel whose waves either stage or multiply;
                  # 17 and 19 slabs leave a ragged end to its look-ahead, C = 1 is not ternary
                  (4096, 512, 2048, 11), (4096, 2048, 512, 11), (4096, 544, 2048, 3), (4096, 2048, 608, 4),
-                 (4096, 640, 2048, 1), (2048, 4096, 1024, 1)]
+                 (4096, 640, 2048, 1), (2048, 4096, 1024, 1),
+                 # a ragged token count over the same kernels: whole 128-row tiles, then the checked kernel
+                 (4100, 512, 2048, 11), (4223, 2048, 512, 3), (200, 256, 128, 11)]
 
 
 @pytest.mark.parametrize("shape", LINEAR_SHAPES, ids=lambda s: "N%d_in%d_out%d_C%d" % s)
