@@ -451,6 +451,20 @@ def bench_update_only(L, ops, steps, warmup, by_row_length=True):
         mean_ms, med_ms = time_steps(lambda i: ops.apply_update_dense_batched(sb, C, LR_SCALE, BETA, EPS), max(steps, 10), 0)
         by_width[str(width)] = {"tensors": len(sub), "ms_per_call": med_ms, "gparam_per_s": sub_params / (med_ms * 1e-3) / 1e9,
                                 "hbm_frac": BYTES_PER_PARAM * sub_params / (med_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    # row lengths of other model sizes (13B: 5120 / 13824, 70B: 8192 / 28672), outside cfg3: the classes of
+    # cooperating waves that rows of 4097..32768 weights take
+    for width in ((5120, 8192, 13824, 28672) if by_row_length else ()):
+        sub = [(make_state(ops, 4096, width), normal(ops, (4096, width), 0.01)) for _ in range(8)]
+        sub = [(st[0], st[1], st[2], g) for (st, g) in sub]
+        sub_params = sum(t[3].numel() for t in sub)
+        sb = ops.UpdateBatch(sub, LR, list(range(len(sub))))
+        for _ in range(30):
+            ops.apply_update_dense_batched(sb, C, LR_SCALE, BETA, EPS)
+        mean_ms, med_ms = time_steps(lambda i: ops.apply_update_dense_batched(sb, C, LR_SCALE, BETA, EPS), max(steps, 10), 0)
+        by_width[str(width)] = {"tensors": len(sub), "shape": [4096, width], "in_cfg3": False, "ms_per_call": med_ms,
+                                "gparam_per_s": sub_params / (med_ms * 1e-3) / 1e9,
+                                "hbm_frac": BYTES_PER_PARAM * sub_params / (med_ms * 1e-3) / 1e9 / PEAK_HBM_GBS}
+        del sub, sb
     out["by_row_length"] = by_width
     out["roofline"]["clock_mhz"] = clock_during(ops, lambda: step(0), ms_per_step)
     return out, tensors
