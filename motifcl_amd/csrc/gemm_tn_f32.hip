@@ -64,9 +64,10 @@ __global__ __launch_bounds__(256) void reduce_slices_kernel(const float* __restr
 // their chunk slices).  A small layer is tens of microseconds of work, so a model made of such
 // layers is bound by launches when every tensor goes out on its own; here the descriptors
 // travel as kernel arguments and a workgroup finds its tensor by scanning their first-workgroup
-// indices.  Each tensor keeps the plan (tile size, chunks) it has on its own, and the register-
-// staged main loop sums in the same order as the direct-to-LDS one, so the gradients are the
-// same bits as from launch_gemm_tn_f32.
+// indices.  The order of a gradient's token sum depends on the token chunks alone, not on the tile
+// size or on how a slab reaches LDS: while every tensor keeps the chunks of its own plan the
+// gradients are the same bits as from launch_gemm_tn_f32; a list whose tiles fill the device is
+// cut into fewer chunks (list_splits), and its gradients are then those sums.
 // ---------------------------------------------------------------------------
 struct GemmGroupItem {
     const float* a;
@@ -112,6 +113,123 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_tn_group_kernel(GemmGroupAr
                 if (row < it.M && col < it.N) c[(size_t)row * it.N + col] = acc[ii][j][r];
             }
         }
+}
+
+// 96 x 96 tiles for the grouped launch: 288- and 768-wide layers (the 15M-shaped model) are whole
+// numbers of them, where 64 x 64 tiles cover 288 as 320 (a fifth of the matrix instructions wasted).
+// Three waves, each 32 rows x 96 columns of the tile: four operand reads per three matrix
+// instructions where the 2 x 2 waves of a 64 x 64 tile need six.  Same slabs, same order of the
+// token sum as the other tiles, so the same bits.  m and n multiples of 96, operands 16-byte
+// aligned.
+constexpr int kThreads96 = 192;
+// DIRECT: every chunk is a whole number of slabs, so the slabs go from global memory straight into
+// one of two unpadded LDS buffers (no staging registers, no LDS store instructions, one barrier per
+// slab); otherwise through registers with the end of a ragged chunk zero-filled.
+template <bool DIRECT>
+__global__ __launch_bounds__(kThreads96) void gemm_tn_group96_kernel(GemmGroupArgs g) {
+    constexpr int kT96 = 96, kLd = DIRECT ? kT96 : kT96 + 4;
+    constexpr int kSlab = kBK * kLd;  // floats of one operand's slab
+    __shared__ float lds[(DIRECT ? 4 : 2) * kSlab];
+    const int wg = blockIdx.x;
+    int i = 0;
+    while (i + 1 < g.n && wg >= g.it[i + 1].wg_start) ++i;  // uniform: scalar loads of the arguments
+    const GemmGroupItem it = g.it[i];
+    const int local = wg - it.wg_start;
+    const int z = local / it.tiles, t = local - z * it.tiles;
+    const int ty = t / it.tiles_x, tx = t - ty * it.tiles_x;
+    const int m0 = ty * kT96, n0 = tx * kT96;
+    const int k_begin = z * it.chunk;
+    const int k_len = it.K - k_begin < it.chunk ? it.K - k_begin : it.chunk;
+    const float* a = it.a + (size_t)k_begin * it.M;
+    const float* b = it.b + (size_t)k_begin * it.N;
+    float* c = it.out + (size_t)z * it.M * it.N;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    floatx16 acc[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+    auto multiply = [&](const float* lds_a, const float* lds_b) {
+#pragma unroll
+        for (int kk = 0; kk < kBK / 2; ++kk) {
+            const int krow = 2 * kk + half;
+            const float fa = lds_a[krow * kLd + 32 * wave + l32];
+            float fb[3];
+#pragma unroll
+            for (int j = 0; j < 3; ++j) fb[j] = lds_b[krow * kLd + 32 * j + l32];
+#pragma unroll
+            for (int j = 0; j < 3; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb[j], acc[j], 0, 0, 0);
+        }
+    };
+    // 16 x 96 floats per operand and slab = 384 float4: two per thread (row = idx / 24, c4 = idx % 24)
+    if constexpr (DIRECT) {
+        typedef __attribute__((address_space(3))) void* lds_ptr;
+        typedef const __attribute__((address_space(1))) void* global_ptr;
+        auto issue = [&](int k0, int buf) {
+            float* dst_a = lds + buf * 2 * kSlab;
+            float* dst_b = dst_a + kSlab;
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int chunk = 3 * p + wave;  // 64 consecutive float4 of the slab
+                const int idx = chunk * 64 + lane;
+                const int row = idx / 24, c4 = idx % 24;
+                __builtin_amdgcn_global_load_lds((global_ptr)(a + (size_t)(k0 + row) * it.M + m0 + 4 * c4),
+                                                 (lds_ptr)(dst_a + chunk * 256), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((global_ptr)(b + (size_t)(k0 + row) * it.N + n0 + 4 * c4),
+                                                 (lds_ptr)(dst_b + chunk * 256), 16, 0, 0);
+            }
+        };
+        issue(0, 0);
+        int buf = 0;
+        for (int k0 = 0; k0 < k_len; k0 += kBK) {
+            __builtin_amdgcn_s_waitcnt(0);  // this wave's part of the slab has landed
+            __syncthreads();                // ... and everybody else's; the other buffer is free
+            if (k0 + kBK < k_len) issue(k0 + kBK, buf ^ 1);
+            multiply(lds + buf * 2 * kSlab, lds + buf * 2 * kSlab + kSlab);
+            buf ^= 1;
+        }
+    } else {
+        float* lds_a = lds;
+        float* lds_b = lds + kSlab;
+        float4 ra[2], rb[2];
+        auto fetch = [&](int k0) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int idx = tid + kThreads96 * p;
+                const int row = idx / 24, c4 = idx % 24;
+                // a slab past the end of a chunk that is not a whole number of slabs is zero-filled
+                const bool in = k0 + row < k_len;
+                ra[p] = in ? *reinterpret_cast<const float4*>(a + (size_t)(k0 + row) * it.M + m0 + 4 * c4)
+                           : make_float4(0.f, 0.f, 0.f, 0.f);
+                rb[p] = in ? *reinterpret_cast<const float4*>(b + (size_t)(k0 + row) * it.N + n0 + 4 * c4)
+                           : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        };
+        fetch(0);
+        for (int k0 = 0; k0 < k_len; k0 += kBK) {
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int idx = tid + kThreads96 * p;
+                const int row = idx / 24, c4 = idx % 24;
+                *reinterpret_cast<float4*>(&lds_a[row * kLd + 4 * c4]) = ra[p];
+                *reinterpret_cast<float4*>(&lds_b[row * kLd + 4 * c4]) = rb[p];
+            }
+            __syncthreads();
+            if (k0 + kBK < k_len) fetch(k0 + kBK);
+            multiply(lds_a, lds_b);
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int col = n0 + 32 * j + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = m0 + 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
+            c[(size_t)row * it.N + col] = acc[j][r];
+        }
+    }
 }
 
 struct ReduceGroupItem {
@@ -290,34 +408,80 @@ hipError_t launch_gemm_tn_f32(hipStream_t stream, const float* a, const float* b
 // The contractions of `n` tensors (c = slice 0 of `out`, which holds gemm_tn_slices floats-matrices).
 // Tensors whose operands are 16-byte aligned with m, n multiples of 4 are grouped by tile size;
 // the others, and very large ones (which fill the device alone), go out one by one.
+// Whether job j can share a grouped launch of `tile`-sized tiles, and its plan on its own.
+// (tile 96: the small-tile plan on 96 x 96 tiles, for sides that are multiples of 96)
+static bool groupable(const GemmTnJob& j, int tile, GemmTnPlan* plan_out, long* tiles_out) {
+    const GemmTnPlan plan = plan_gemm_tn(j.k, j.m, j.n);
+    const bool vec = j.m % 4 == 0 && j.n % 4 == 0 && (reinterpret_cast<uintptr_t>(j.a) & 15u) == 0 &&
+                     (reinterpret_cast<uintptr_t>(j.b) & 15u) == 0;
+    const bool fits96 = plan.tile == 64 && j.m % 96 == 0 && j.n % 96 == 0;
+    const int side = tile == 96 ? 96 : plan.tile;
+    const long tiles = (long)((j.m + side - 1) / side) * ((j.n + side - 1) / side);
+    *plan_out = plan;
+    *tiles_out = tiles;
+    if (tile == 96 ? !fits96 : (plan.tile != tile || fits96)) return false;
+    // a tensor of 1024 workgroups or more gains nothing from sharing a launch, and one whose
+    // chunks fill the device with wide tiles is faster on those
+    if (!vec || tiles * plan.splits >= 1024) return false;
+    if (plan.tile == 128 && gemm_tn_wide_supports(j.a, j.b, j.k, j.m, j.n, plan.chunk) &&
+        wide_chunks_fill_the_device(j.m, j.n, plan.splits))
+        return false;
+    return true;
+}
+
+// Token chunks of a list: a tensor's own plan cuts its tokens until its tiles alone fill the device
+// (32 chunks for a 288 x 288 layer), which is slices to write and to add.  When the tiles of the
+// whole list of one class fill the device twice over, the list is cut instead: as many chunks as
+// bring the list to about sixteen workgroups a CU, the same for every tensor (0: keep the tensors'
+// own plans; measured flat from 13 to 24 a CU).  15M-shaped model, 42 tensors: six chunks of 96 x 96 tiles.
+static int list_splits(const GemmTnJob* jobs, size_t n, int tile) {
+    long total = 0;
+    for (size_t i = 0; i < n; ++i) {
+        GemmTnPlan plan;
+        long tiles;
+        if (groupable(jobs[i], tile, &plan, &tiles)) total += tiles;
+    }
+    if (total < 512) return 0;  // two tiles for each of the 256 CUs
+    const long s = 4096 / total;
+    return s < 1 ? 1 : (int)s;
+}
+
 hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_t n) {
     std::vector<char> grouped(n, 0);
-    for (int tile : {64, 128}) {
+    std::vector<int> splits_used(n, 0);
+    for (int tile : {96, 64, 128}) {
+        const int of_list = list_splits(jobs, n, tile);
         GemmGroupArgs g;
         g.n = 0;
         int wgs = 0;
+        bool whole_slabs = true;  // of the descriptors gathered so far: every chunk a whole number of slabs
         auto flush = [&]() -> hipError_t {
             if (g.n == 0) return hipSuccess;
-            if (tile == 64)
+            if (tile == 96 && whole_slabs)
+                hipLaunchKernelGGL(gemm_tn_group96_kernel<true>, dim3(wgs), dim3(kThreads96), 0, stream, g);
+            else if (tile == 96)
+                hipLaunchKernelGGL(gemm_tn_group96_kernel<false>, dim3(wgs), dim3(kThreads96), 0, stream, g);
+            else if (tile == 64)
                 hipLaunchKernelGGL((gemm_tn_group_kernel<64, 64>), dim3(wgs), dim3(kGemmThreads), 0, stream, g);
             else
                 hipLaunchKernelGGL((gemm_tn_group_kernel<128, 128>), dim3(wgs), dim3(kGemmThreads), 0, stream, g);
             g.n = 0;
             wgs = 0;
+            whole_slabs = true;
             return hipGetLastError();
         };
         for (size_t i = 0; i < n; ++i) {
             const GemmTnJob& j = jobs[i];
-            const GemmTnPlan plan = plan_gemm_tn(j.k, j.m, j.n);
-            const bool vec = j.m % 4 == 0 && j.n % 4 == 0 && (reinterpret_cast<uintptr_t>(j.a) & 15u) == 0 &&
-                             (reinterpret_cast<uintptr_t>(j.b) & 15u) == 0;
-            const long tiles = (long)((j.m + plan.tile - 1) / plan.tile) * ((j.n + plan.tile - 1) / plan.tile);
-            // a tensor of 1024 workgroups or more gains nothing from sharing a launch, and one whose
-            // chunks fill the device with wide tiles is faster on those
-            if (plan.tile != tile || !vec || tiles * plan.splits >= 1024) continue;
-            if (plan.tile == 128 && gemm_tn_wide_supports(j.a, j.b, j.k, j.m, j.n, plan.chunk) &&
-                wide_chunks_fill_the_device(j.m, j.n, plan.splits))
-                continue;
+            GemmTnPlan plan;
+            long tiles;
+            if (!groupable(j, tile, &plan, &tiles)) continue;
+            if (of_list > 0 && of_list < plan.splits) {  // (never more slices than the tensor's region holds)
+                const int chunk = (j.k + of_list - 1) / of_list;
+                plan.chunk = (chunk + kBK - 1) / kBK * kBK;
+                plan.splits = (j.k + plan.chunk - 1) / plan.chunk;
+            }
+            splits_used[i] = plan.splits;
+            if (j.k % kBK != 0 || plan.chunk % kBK != 0) whole_slabs = false;
             if (g.n == kMaxGemmGroup || wgs > (1 << 30)) {
                 const hipError_t e = flush();
                 if (e != hipSuccess) return e;
@@ -355,9 +519,7 @@ hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_
         return hipGetLastError();
     };
     for (size_t i = 0; i < n; ++i) {
-        if (!grouped[i]) continue;
-        const GemmTnPlan plan = plan_gemm_tn(jobs[i].k, jobs[i].m, jobs[i].n);
-        if (plan.splits == 1) continue;
+        if (!grouped[i] || splits_used[i] == 1) continue;
         if (r.n == kMaxReduceGroup) {
             const hipError_t e = flush_reduce();
             if (e != hipSuccess) return e;
@@ -365,7 +527,7 @@ hipError_t launch_gemm_tn_group(hipStream_t stream, const GemmTnJob* jobs, size_
         ReduceGroupItem& it = r.it[r.n++];
         it.slices = jobs[i].out;
         it.mn = (unsigned)((size_t)jobs[i].m * jobs[i].n);  // below 2^32: the tensor has fewer than 1024 tiles
-        it.n_slices = plan.splits;
+        it.n_slices = splits_used[i];
         it.block_start = blocks;
         it.pad = 0;
         blocks += (int)((it.mn + kReduceBlockElems - 1) / kReduceBlockElems);

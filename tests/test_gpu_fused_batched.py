@@ -101,11 +101,14 @@ def test_list_of_256_multiple_layers_runs_as_equal_spans_with_the_same_bytes(ops
             np.testing.assert_array_equal(host(got), want)
 
 
-def test_equal_spans_over_a_list_against_the_oracle(ops, oracle):
+@pytest.mark.parametrize("model", [(768, 2048, 12), (288, 768, 6)], ids=["110m_equal_spans", "15m_small_tiles"])
+def test_equal_spans_over_a_list_against_the_oracle(ops, oracle, model):
     # 1024 tokens: the per-tensor call would split them into chunks; the list's gradients are the
-    # unchunked sums.  Each gradient within 1e-4 of the oracle's sequential sum, state / scale / v
-    # exact for the GPU's gradient, counter flips against the sequential-sum oracle counted.
-    shapes = layer_shapes(768, 2048, 12, 1024)
+    # unchunked sums (equal spans of 256 x 256 tiles for the 110M shapes; for the 15M shapes the
+    # list's 1680 small tiles fill the device, so nothing is chunked either).  Each gradient within
+    # 1e-4 of the oracle's sequential sum, state / scale / v exact for the GPU's gradient, counter
+    # flips against the sequential-sum oracle counted.
+    shapes = layer_shapes(*model, 1024)
     host_tensors = build(ops, oracle, shapes, 33)
     seeds = [4000 + i for i in range(len(shapes))]
     d_all = [[dev(t) for t in tensor] for tensor in host_tensors]
@@ -116,7 +119,9 @@ def test_equal_spans_over_a_list_against_the_oracle(ops, oracle):
     offset, n_flip, n_all = 0, 0, 0
     for (state, scale, v, dy, x), seed, (n_out, n_in, tokens), d in zip(host_tensors, seeds, shapes, d_all):
         g_gpu = ws[offset: offset + n_out * n_in * 4].view(torch.float32).view(n_out, n_in).cpu().numpy()
-        offset += (n_out * n_in * 4 + 255) // 256 * 256
+        # a tensor's region of the workspace: its gradient alone under equal spans, else what its own call asks for
+        region = n_out * n_in * 4 if model[0] % 256 == 0 else ops.fused_workspace_nbytes(n_in, n_out, tokens)
+        offset += (region + 255) // 256 * 256
         e_state, e_scale, e_v, g_seq = oracle.update_fused(state, scale, v, dy, x, HP["C"], HP["lr"], 0.0,
                                                           HP["rms_beta"], HP["rms_eps"], seed)
         assert np.abs(g_gpu - g_seq).max() <= 1e-4 * np.abs(g_seq).max()
@@ -128,7 +133,7 @@ def test_equal_spans_over_a_list_against_the_oracle(ops, oracle):
         diff = oracle.unpack_codes(x_state) != oracle.unpack_codes(e_state)
         n_flip += int(diff.sum())
         n_all += diff.size
-    print("equal spans over 84 tensors at 1024 tokens: counter-flip fraction vs the sequential-sum oracle %.2e" % (n_flip / n_all))
+    print("%d tensors at 1024 tokens, unchunked: counter-flip fraction vs the sequential-sum oracle %.2e" % (len(shapes), n_flip / n_all))
     assert n_flip / n_all <= 1e-4
 
 
