@@ -18,8 +18,9 @@
 // line multiplies by the scale first, as kernels/compact_counter.cl:262-267 does).  Non-finite
 // activations are outside this kernel's contract (inf - inf in the split).
 //
-// Tile: 128 rows x 128 or 256 columns per workgroup of 4 or 8 waves (64 x 64 each), 32-deep
-// slabs.  LDS holds the three activation planes and the weight tile as [row][32 bf16] = 64-byte
+// Tile: 128 rows x 128 or 256 columns per workgroup, 32-deep slabs: 4 or 8 waves of 64 x 64 that
+// each stage and multiply (counter_linear_bf16x3_kernel), or, for large products, 16 waves of
+// which half stage and half multiply (counter_linear_bf16x3_split_roles_kernel).  LDS holds the three activation planes and the weight tile as [row][32 bf16] = 64-byte
 // rows whose four 16-byte chunks are XOR-swizzled with bits 2-3 of the row, which makes the
 // 16-byte MFMA operand reads (lane = row, 8 consecutive k) conflict-free without padding:
 // 32 or 40 KiB per workgroup.  Splitting and decoding are done by the thread that fetched the
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 3 : 4) void counter_linear_bf16
 // them: 8 activations and 4 packed groups per thread), two of each kind on every SIMD.  In the
 // kernel above every wave stages and then multiplies, the waves of a SIMD do so in step, and the
 // matrix pipe idles while they stage (busy 54 % of the cycles); here the SIMD's matrix pipe and
-// its vector ALUs work at the same time on different waves (68 %).  Two LDS buffers (the stagers
+// its vector ALUs work at the same time on different waves (67-72 %).  Two LDS buffers (the stagers
 // fill one while the other is multiplied), one barrier per slab.  What made the difference, in
 // the order found:
 //   - nothing computed from a loaded value inside the fetch (it would wait for the load there),
