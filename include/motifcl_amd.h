@@ -231,6 +231,11 @@ int mcc_compact_counter_apply_update_fused_static(
  * wherever that call does not split the tokens into chunks and differ from it
  * by the rounding of its chunk sums elsewhere (counter-flip fraction ~1e-6).
  * Such a list needs 16-byte aligned grad_out and x.
+ * Likewise a list of small layers whose tiles together number 512 or more (the
+ * 15M-shaped model: 42 layers) is cut into token chunks per list, fewer than a
+ * layer's own call would use: its gradients are the sums over those chunks,
+ * state, scale and v exact for them, with the same relation to the per-tensor
+ * call.
  * `workspace` (256-byte aligned) holds
  * mcc_compact_counter_fused_batched_workspace_nbytes(tensors, n) bytes: the
  * per-tensor workspaces, each rounded up to 256 bytes, one after the other (as
